@@ -1,0 +1,30 @@
+"""CPU/GPU-agnostic plain-torch restatement of the reference's attention operators.
+
+TEST INFRASTRUCTURE ONLY.  Nothing in the shipped package imports this directory: it is the
+checker used by ``tests/``, by ``__graft_entry__.smoke()`` and by the ``cpu_baseline`` leg of
+``bench.py``.  The product path (``flagattention_amd``) calls hand-written HIP kernels through a
+C-ABI library and raises when that library is missing.
+
+Each function follows one file of the reference's PyTorch restatements
+(``src/flag_attn/testing/{flash,piecewise,paged}.py``) and cites the lines it follows.
+
+How each function is pinned (the reference ships no golden vectors, every one of its tests is a
+randomized three-way comparison), see ``tests/test_oracle_*.py``:
+
+* ``flash_attention``: ``torch.nn.functional.scaled_dot_product_attention`` (non-causal, and
+  causal with equal lengths), an explicit fp64 triple loop on tiny inputs (bottom-right causal
+  alignment, empty rows), ``torch.logsumexp`` for the log-normalizer, column sums and the
+  ``sum_n tot[n] == number of non-empty rows`` invariant for total attention, GQA == MHA on
+  repeated heads, closed-form gradients and ``torch.autograd.gradcheck`` in fp64.
+* ``piecewise_attention``: reduces to ``flash_attention`` when both (q, k) pairs are equal, when
+  the threshold exceeds every distance, when it is below every distance; fp64 loop on tiny inputs;
+  closed-form gradients (``src/flag_attn/testing/piecewise.py:36-78``).
+* ``paged_attention``: equals dense single-query attention on the gathered keys/values, invariant
+  under a permutation of the cache blocks with the block table permuted alike; fp64 loop.
+
+No function of this oracle is "parity unpinned".
+"""
+from .flash import flash_attention  # noqa: F401
+from .piecewise import piecewise_attention, piecewise_attention_grad  # noqa: F401
+from .paged import paged_attention  # noqa: F401
+from .compare import max_abs_diff, within_two_x  # noqa: F401
