@@ -1,0 +1,257 @@
+// FlashAttention-2 forward for gfx950, and its piecewise (two score regimes) variant.
+//
+// Replaces the reference's Triton kernels `_fwd_kernel` (src/flag_attn/flash.py:325-489) and the
+// piecewise `_fwd_kernel` (src/flag_attn/piecewise.py:223-370).
+//
+// Work decomposition: one workgroup (4 wavefronts) owns 128 query rows of one (batch, head); each
+// wavefront owns 32 of them and keeps, for the whole kernel,
+//   * its Q rows as the B operand of S^T = K Q^T (registers, never in LDS),
+//   * O^T (D x 32) as fp32 accumulators,
+//   * the running row maximum and the lane-partial row sum of the online softmax.
+// Working on S^T puts one query row in one lane (and its lane^32 twin), so the row maximum and row
+// sum are register reductions plus one cross-lane exchange, and the probabilities come out of the
+// first product already in the operand layout of the second (O^T = V^T P^T) -- no LDS round trip.
+// K/V tiles of 64 keys are staged global -> registers -> LDS, double buffered, with the next tile's
+// global loads in flight during the current tile's matrix work.  V is read from LDS through the
+// transposing 64-bit read.
+#include "common.hpp"
+#include "params.hpp"
+
+namespace fa {
+
+template <class T, int D, bool PW>
+struct FwdCfg {
+  static constexpr int BM = 128, BN = 64;
+  static constexpr int DV = D < 32 ? 32 : D;  // value/output width rounded up to one MFMA block
+  static constexpr int KSTEPS = D / 16;
+  static constexpr int K_LD = D + 8;    // 16 B of padding: conflict-free 16-byte row reads
+  static constexpr int V_LD = DV + 32;  // 64 B of padding: the 4 rows of a transposing read fall in disjoint banks
+  static constexpr int K_TILE = BN * K_LD, V_TILE = BN * V_LD;
+  static constexpr int STAGE = (PW ? 2 : 1) * K_TILE + V_TILE;  // elements per pipeline stage
+  static constexpr size_t LDS_BYTES = 2 * STAGE * sizeof(T);
+};
+
+template <class T, int D, bool PW>
+FA_KERNEL void FA_LAUNCH_BOUNDS(kThreads) fa_fwd_kernel(FwdParams p) {
+  using C = FwdCfg<T, D, PW>;
+  using V8 = typename hw::Elem<T>::v8;
+  FA_LDS_DECL(smem);
+  T* lds = (T*)smem;
+
+  const int tid = hw::thread_id(), lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, hh = lane >> 5;
+  const int mb = hw::grid_x() - 1 - hw::block_x();  // long rows first under the causal mask
+  const int head = hw::block_y(), batch = hw::block_z();
+  const int hk = head / p.group;
+  const int M = p.M, N = p.N, pseq = N - M;
+  const int m0 = mb * C::BM, mw = m0 + wave * 32, my_m = mw + l32;
+
+  const T* qb = (const T*)p.q.ptr + batch * p.q.sb + head * p.q.sh;
+  const T* kb = (const T*)p.k.ptr + batch * p.k.sb + hk * p.k.sh;
+  const T* vb = (const T*)p.v.ptr + batch * p.v.sb + hk * p.v.sh;
+  const T* q2b = PW ? (const T*)p.q2.ptr + batch * p.q2.sb + head * p.q2.sh : nullptr;
+  const T* k2b = PW ? (const T*)p.k2.ptr + batch * p.k2.sb + hk * p.k2.sh : nullptr;
+
+  // ---- Q (and Q2) rows of this lane as B operands: k = 16 * kk + 8 * hh + 0..7 ----
+  V8 qreg[C::KSTEPS], q2reg[PW ? C::KSTEPS : 1];
+#pragma unroll
+  for (int kk = 0; kk < C::KSTEPS; ++kk) {
+    u32x4 z = {0u, 0u, 0u, 0u}, z2 = {0u, 0u, 0u, 0u};
+    if (my_m < M) {
+      z = *(const u32x4*)(qb + (int64_t)my_m * p.q.st + 16 * kk + 8 * hh);
+      if (PW) z2 = *(const u32x4*)(q2b + (int64_t)my_m * p.q2.st + 16 * kk + 8 * hh);
+    }
+    qreg[kk] = hw::as_v8<T>(z);
+    if (PW) q2reg[kk] = hw::as_v8<T>(z2);
+  }
+
+  // ---- key range of this workgroup ----
+  int hi = N;
+  if (p.causal) hi = imin(N, pseq + m0 + C::BM);
+  const int n_tiles = hi > 0 ? cdiv(hi, C::BN) : 0;
+
+  // When D < 32 the value tile has columns D..31 that no load ever writes: clear both stages once.
+  if (C::DV != D) {
+    for (int i = tid; i < 2 * C::STAGE; i += kThreads) lds[i] = (T)0.f;
+    hw::block_sync();
+  }
+
+  const float c2 = p.sm_scale * kLog2e;
+  float m_i = neg_inf(), l_i = 0.f;
+  f32x16 oacc[C::DV / 32];
+#pragma unroll
+  for (int i = 0; i < C::DV / 32; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) oacc[i][r] = 0.f;
+
+  // Which key tiles need which (q, k) pair: pair 2 serves distance >= w, pair 1 distance < w.
+  // Over the workgroup's rows and a tile's keys the distance m + pseq - n spans
+  //   [m0 + pseq - (n0 + BN - 1), m0 + BM - 1 + pseq - n0].
+  auto tile_needs_near = [&](int n0) { return !PW || (m0 + pseq - (n0 + C::BN - 1) < p.w); };
+  auto tile_needs_far = [&](int n0) { return PW && (m0 + C::BM - 1 + pseq - n0 >= p.w); };
+
+  TileRegs<C::BN, D> kr, vr, k2r;
+  auto fetch = [&](int n0) {
+    if (tile_needs_near(n0)) tile_fetch<T, C::BN, D>(kr, kb, p.k.st, n0, N, tid);
+    if (tile_needs_far(n0)) tile_fetch<T, C::BN, D>(k2r, k2b, p.k2.st, n0, N, tid);
+    tile_fetch<T, C::BN, D>(vr, vb, p.v.st, n0, N, tid);
+  };
+  auto commit = [&](int n0, int stage) {
+    T* s = lds + stage * C::STAGE;
+    if (tile_needs_near(n0)) tile_commit<T, C::BN, D, C::K_LD>(kr, s, tid);
+    if (tile_needs_far(n0)) tile_commit<T, C::BN, D, C::K_LD>(k2r, s + C::K_TILE, tid);
+    tile_commit<T, C::BN, D, C::V_LD>(vr, s + (PW ? 2 : 1) * C::K_TILE, tid);
+  };
+
+  if (n_tiles > 0) {
+    fetch(0);
+    commit(0, 0);
+  }
+  hw::block_sync();
+
+  for (int it = 0; it < n_tiles; ++it) {
+    const int n0 = it * C::BN;
+    const bool more = it + 1 < n_tiles;
+    if (more) fetch(n0 + C::BN);
+
+    const T* sK = lds + (it & 1) * C::STAGE;
+    const T* sK2 = sK + C::K_TILE;
+    const T* sV = sK + (PW ? 2 : 1) * C::K_TILE;
+
+    // ---- S^T = K Q^T : BN/32 blocks of (32 keys x 32 queries) ----
+    f32x16 s[C::BN / 32];
+#pragma unroll
+    for (int nb = 0; nb < C::BN / 32; ++nb) {
+      const int nlo = n0 + nb * 32;
+      bool near = true, far = false;
+      if (PW) {  // wavefront-uniform: distances over this 32 x 32 block
+        near = (mw + pseq - (nlo + 31)) < p.w;
+        far = (mw + 31 + pseq - nlo) >= p.w;
+      }
+      f32x16 a1, a2;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { a1[r] = 0.f; a2[r] = 0.f; }
+      if (near) {
+#pragma unroll
+        for (int kk = 0; kk < C::KSTEPS; ++kk)
+          a1 = hw::mfma32(operand_rowmajor<T, C::K_LD>(sK, nb * 32, 16 * kk, lane), qreg[kk], a1);
+      }
+      if (PW && far) {
+#pragma unroll
+        for (int kk = 0; kk < C::KSTEPS; ++kk)
+          a2 = hw::mfma32(operand_rowmajor<T, C::K_LD>(sK2, nb * 32, 16 * kk, lane), q2reg[kk], a2);
+      }
+      if (PW) {
+        if (far && near) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            int n = nlo + block_row(r, hh);
+            a1[r] = (my_m + pseq - n >= p.w) ? a2[r] : a1[r];
+          }
+        } else if (far) {
+          a1 = a2;
+        }
+      }
+      s[nb] = a1;
+    }
+
+    // ---- masks (key tail, causal) only on tiles that need them ----
+    const bool need_mask = (n0 + C::BN > N) || (p.causal && (n0 + C::BN - 1 > pseq + mw));
+    if (need_mask) {
+#pragma unroll
+      for (int nb = 0; nb < C::BN / 32; ++nb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          int n = n0 + nb * 32 + block_row(r, hh);
+          bool keep = (n < N) && (!p.causal || (my_m + pseq >= n));
+          s[nb][r] = keep ? s[nb][r] : neg_inf();
+        }
+    }
+
+    // ---- online softmax (base 2); a query row lives in lanes l and l ^ 32 ----
+    float mx = neg_inf();
+#pragma unroll
+    for (int nb = 0; nb < C::BN / 32; ++nb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[nb][r]);
+    mx = fmaxf(mx, hw::xor32(mx));
+    const float m_new = fmaxf(m_i, mx);
+    const float m_use = (m_new == neg_inf()) ? 0.f : m_new;  // row with no visible key so far
+    const float alpha = hw::exp2_fast((m_i - m_use) * c2);
+    const float shift = -m_use * c2;
+    float psum = 0.f;
+#pragma unroll
+    for (int nb = 0; nb < C::BN / 32; ++nb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        float e = hw::exp2_fast(fmaf(s[nb][r], c2, shift));
+        s[nb][r] = e;
+        psum += e;
+      }
+    l_i = l_i * alpha + psum;
+    m_i = m_new;
+#pragma unroll
+    for (int i = 0; i < C::DV / 32; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
+
+    // ---- O^T += V^T P^T ; P is rounded to the input dtype as the reference does ----
+#pragma unroll
+    for (int nb = 0; nb < C::BN / 32; ++nb)
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        V8 pb = pack_half_block<T>(s[nb], c);
+#pragma unroll
+        for (int db = 0; db < C::DV / 32; ++db)
+          oacc[db] = hw::mfma32(operand_transposed<T, C::V_LD>(sV, nb * 32 + 16 * c, db * 32, lane), pb, oacc[db]);
+      }
+
+    if (more) commit(n0 + C::BN, (it + 1) & 1);
+    hw::block_sync();
+  }
+
+  // ---- epilogue: O = acc / l, L = m * scale + ln(l); rows that saw no key give O = 0, L = -inf ----
+  const float l_tot = l_i + hw::xor32(l_i);
+  const bool empty = !(l_tot > 0.f);
+  const float inv = empty ? 0.f : 1.f / l_tot;
+  if (my_m < M) {
+    T* ob = (T*)p.o.ptr + batch * p.o.sb + head * p.o.sh + (int64_t)my_m * p.o.st;
+#pragma unroll
+    for (int db = 0; db < C::DV / 32; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        int d = db * 32 + 8 * g + 4 * hh;
+        if (d < D) {
+          hw::u32x2 w;
+          w[0] = (uint32_t)hw::bits16<T>(oacc[db][4 * g + 0] * inv) | ((uint32_t)hw::bits16<T>(oacc[db][4 * g + 1] * inv) << 16);
+          w[1] = (uint32_t)hw::bits16<T>(oacc[db][4 * g + 2] * inv) | ((uint32_t)hw::bits16<T>(oacc[db][4 * g + 3] * inv) << 16);
+          *(hw::u32x2*)(ob + d) = w;
+        }
+      }
+    if (hh == 0)
+      p.lse[((int64_t)batch * p.H + head) * M + my_m] = empty ? neg_inf() : m_i * p.sm_scale + hw::log_nat(l_tot);
+  }
+}
+
+template <class T, bool PW>
+static int launch_fwd(const FwdParams& p, hipStream_t stream) {
+  dim3 grid((p.M + 127) / 128, p.H, p.B);
+  switch (p.D) {
+    case 16: return launch(fa_fwd_kernel<T, 16, PW>, grid, FwdCfg<T, 16, PW>::LDS_BYTES, stream, p);
+    case 32: return launch(fa_fwd_kernel<T, 32, PW>, grid, FwdCfg<T, 32, PW>::LDS_BYTES, stream, p);
+    case 64: return launch(fa_fwd_kernel<T, 64, PW>, grid, FwdCfg<T, 64, PW>::LDS_BYTES, stream, p);
+    case 128: return launch(fa_fwd_kernel<T, 128, PW>, grid, FwdCfg<T, 128, PW>::LDS_BYTES, stream, p);
+  }
+  return kUnsupported;
+}
+
+int run_fwd(const FwdParams& p, bool piecewise, hipStream_t stream) {
+  if (p.B <= 0 || p.H <= 0 || p.M <= 0 || p.N < 0 || p.group <= 0) return kBadArgument;
+  if (p.dtype == kDtypeF16)
+    return piecewise ? launch_fwd<hw::half_t, true>(p, stream) : launch_fwd<hw::half_t, false>(p, stream);
+  if (p.dtype == kDtypeBF16)
+    return piecewise ? launch_fwd<hw::bf16_t, true>(p, stream) : launch_fwd<hw::bf16_t, false>(p, stream);
+  return kUnsupported;
+}
+
+}  // namespace fa

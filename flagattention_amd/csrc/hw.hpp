@@ -1,0 +1,106 @@
+// Thin layer over the gfx950 (CDNA4) instructions the attention kernels are built from.
+//
+// Every kernel in this directory reaches the hardware only through the functions declared here:
+// 64-lane wavefronts, v_mfma_f32_32x32x16_{f16,bf16}, ds_read_b64_tr_b16, a lane^32 exchange and
+// v_exp_f32.  The operand layouts documented below were checked on an MI355X with one-off probes.
+//
+// A second implementation of the same functions (tests/sim/hw_sim.hpp, selected by
+// FLAGATTN_HOST_SIM) runs the unchanged kernel sources lane by lane on the host, with bounds-checked
+// memory, so that index arithmetic can be debugged without a GPU.  It is test infrastructure; the
+// shipped library is always built from the gfx950 half of this file.
+#pragma once
+#include <stdint.h>
+
+#ifdef FLAGATTN_HOST_SIM
+#include "hw_sim.hpp"
+#else
+#include <hip/hip_runtime.h>
+
+namespace hw {
+
+using half_t = _Float16;
+using bf16_t = __bf16;
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef short short8v __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+#define FA_DEVICE __device__ __forceinline__
+#define FA_KERNEL __global__
+#define FA_LAUNCH_BOUNDS(n) __launch_bounds__(n)
+#define FA_LDS_DECL(name) extern __shared__ __attribute__((aligned(16))) unsigned char name[]
+
+FA_DEVICE int thread_id() { return (int)threadIdx.x; }
+FA_DEVICE int block_x() { return (int)blockIdx.x; }
+FA_DEVICE int block_y() { return (int)blockIdx.y; }
+FA_DEVICE int block_z() { return (int)blockIdx.z; }
+FA_DEVICE int grid_x() { return (int)gridDim.x; }
+FA_DEVICE void block_sync() { __syncthreads(); }
+
+// D(32x32) += A(32x16) * B(16x32).  Lane l holds, for h = l / 32:
+//   A[i = l % 32][k = 8h + e], e = 0..7          B[k = 8h + e][j = l % 32]
+//   D[i = 8 * (r / 4) + 4h + r % 4][j = l % 32], r = 0..15
+FA_DEVICE f32x16 mfma32(half8 a, half8 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+}
+FA_DEVICE f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+// D(16x16) += A(16x32) * B(32x16).  Lane l holds, for q = l / 16:
+//   A[i = l % 16][k = 8q + e]     B[k = 8q + e][j = l % 16]     D[i = 4q + r][j = l % 16], r = 0..3
+FA_DEVICE f32x4 mfma16(half8 a, half8 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+}
+FA_DEVICE f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+// Transposing 64-bit LDS read over 16-bit elements.  Within each group of 16 lanes, lane i passes
+// the address of 4 consecutive elements in[i][0..3] and receives
+//   out[i][e] = in[4e + i / 4][i % 4],  e = 0..3
+// i.e. if lane c points at row c / 4, columns 4 * (c % 4).. of a row-major 4 x 16 patch, lane i gets
+// column i of that patch.
+FA_DEVICE short4v lds_read_tr16(const void* lds_ptr) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      (__attribute__((address_space(3))) short4v*)(uintptr_t)lds_ptr);
+}
+
+// Value held by lane (l ^ 32).
+FA_DEVICE float xor32(float x) { return __shfl_xor(x, 32, 64); }
+// Value held by lane (l ^ mask) for mask < 64.
+FA_DEVICE float shfl_xor(float x, int mask) { return __shfl_xor(x, mask, 64); }
+
+FA_DEVICE float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
+FA_DEVICE float log_nat(float x) { return __logf(x); }
+
+}  // namespace hw
+#endif  // FLAGATTN_HOST_SIM
+
+namespace hw {
+
+template <class T> struct Elem;
+template <> struct Elem<half_t> { using v8 = half8; };
+template <> struct Elem<bf16_t> { using v8 = bf16x8; };
+
+// 16 bytes of raw bits <-> 8 elements
+template <class T> FA_DEVICE typename Elem<T>::v8 as_v8(u32x4 raw) {
+  return __builtin_bit_cast(typename Elem<T>::v8, raw);
+}
+template <class T> FA_DEVICE typename Elem<T>::v8 join_v8(short4v lo, short4v hi) {
+  short8v s = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  return __builtin_bit_cast(typename Elem<T>::v8, s);
+}
+template <class T> FA_DEVICE uint16_t bits16(float x) {
+  T t = (T)x;
+  return __builtin_bit_cast(uint16_t, t);
+}
+template <class T> FA_DEVICE float from_bits16(uint16_t b) {
+  return (float)__builtin_bit_cast(T, b);
+}
+
+}  // namespace hw

@@ -1,0 +1,64 @@
+// Plain-data argument blocks passed by value to the kernels, and the internal entry points that the
+// C interface (capi.cpp, include/flagattn.h) forwards to.
+#pragma once
+#include <stdint.h>
+
+namespace fa {
+
+// (batch, head, token, D) view: element strides, unit stride on D.
+struct View4 {
+  const void* ptr;
+  int64_t sb, sh, st;
+};
+
+struct FwdParams {
+  View4 q, k, v, q2, k2;  // q2/k2 only for the piecewise variant
+  View4 o;                // written
+  float* lse;             // (B, H, M) contiguous, natural-log normalizer
+  int B, H, M, N, D;
+  int group;              // query heads per key/value head
+  int causal;
+  int w;                  // piecewise distance threshold
+  float sm_scale;
+  int dtype;
+};
+
+struct BwdParams {
+  View4 q, k, v, q2, k2, o, dout;
+  View4 dq, dk, dv, dq2, dk2;  // written; dk/dv have one slice per *query* head
+  const float* lse;            // (B, H, M)
+  float* delta;                // (B, H, M) rowsum(O * dO): written by the preprocess, read by the rest
+  int B, H, M, N, D;
+  int group;
+  int causal;
+  int w;
+  float sm_scale;
+  int dtype;
+};
+
+struct TotalParams {
+  View4 q, k;
+  const float* lse;  // (B, H, M)
+  float* total;      // (B, H, N)
+  int B, H, M, N, D;
+  int group;
+  int causal;
+  float sm_scale;
+  int dtype;
+};
+
+}  // namespace fa
+
+#ifdef FLAGATTN_HOST_SIM
+typedef void* hipStream_t;
+#else
+#include <hip/hip_runtime.h>
+#endif
+
+namespace fa {
+int run_fwd(const FwdParams& p, bool piecewise, hipStream_t stream);
+int run_bwd_delta(const BwdParams& p, hipStream_t stream);
+int run_bwd_dkdv(const BwdParams& p, bool piecewise, hipStream_t stream);
+int run_bwd_dq(const BwdParams& p, bool piecewise, hipStream_t stream);
+int run_total(const TotalParams& p, hipStream_t stream);
+}  // namespace fa

@@ -1,0 +1,139 @@
+/*
+ * C interface of libflagattn_hip.so: hand-written gfx950 (MI355X) attention kernels behind the
+ * flag_attn operator API.
+ *
+ * Every entry point enqueues its kernels on `stream` (a hipStream_t, passed as void*) of the
+ * current device and returns without synchronizing.  The library never allocates or frees device
+ * memory: outputs and workspaces are caller-owned.  Return value: 0 on success, a negative
+ * FA_ERR_* code for a rejected argument, a positive hipError_t if a launch failed.
+ *
+ * Tensors are described by fa_view4: a device pointer and element strides of a
+ * (batch, head, token, D) view whose D stride is 1.  Pointers must be 16-byte aligned and the three
+ * strides multiples of 8 elements.  `dtype` is FA_F16 or FA_BF16 and applies to every 16-bit tensor
+ * of the call; log-normalizer, delta, total-attention and partial-softmax buffers are fp32.
+ *
+ * Each declaration cites the interface of the reference (FlagOpen/FlagAttention, Triton) that it
+ * replaces.
+ */
+#ifndef FLAGATTN_H
+#define FLAGATTN_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FA_F16 0
+#define FA_BF16 1
+
+#define FA_ERR_BAD_ARGUMENT (-1)
+#define FA_ERR_UNSUPPORTED (-2)
+
+typedef struct fa_view4 {
+  void* ptr;
+  int64_t stride_b, stride_h, stride_t; /* in elements */
+} fa_view4;
+
+/* Library facts. */
+int fa_version(void);
+/* Number of compute units of the current device (the reference reads
+ * torch.cuda.get_device_properties(...).multi_processor_count, src/flag_attn/flash.py:47-48). */
+int fa_num_cus(void);
+
+/* ------------------------------------------------------------------ flash attention, forward --
+ * Replaces the launch of `_fwd_kernel` in FlashAttention.forward, src/flag_attn/flash.py:64-87
+ * (kernel: flash.py:325-489).
+ * q (B, H, M, D); k, v (B, Hk, N, D); o (B, H, M, D) written; lse (B, H, M) contiguous fp32 written
+ * (natural-log normalizer of sm_scale * scores).  H % Hk == 0.  D in {16, 32, 64, 128}.
+ * Causal masking is aligned bottom-right: row m sees key n iff m + N - M >= n; rows that see no key
+ * get o = 0 and lse = -inf. */
+int fa_fwd(int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v, const fa_view4* o,
+           float* lse, int B, int H, int Hk, int M, int N, int D, int causal, float sm_scale,
+           void* stream);
+
+/* ----------------------------------------------------------------- flash attention, backward --
+ * The reference's three launches in FlashAttention.backward, src/flag_attn/flash.py:191-249:
+ *
+ * fa_bwd_delta  <- `_bwd_preprocess` (flash.py:522-568): delta[b,h,m] = sum_d o * dout, fp32.
+ * fa_bwd_dkdv   <- `_bwd_kv_kernel`  (flash.py:571-745): dk, dv of shape (B, H, N, D), one slice per
+ *                  QUERY head; the caller sums groups of H / Hk slices (flash.py:250-251).
+ * fa_bwd_dq     <- `_bwd_q_kernel`   (flash.py:748-909): dq (B, H, M, D), every element written.
+ * No atomics; each workgroup owns its output tile. */
+int fa_bwd_delta(int dtype, const fa_view4* o, const fa_view4* dout, float* delta, int B, int H,
+                 int M, int D, void* stream);
+int fa_bwd_dkdv(int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v,
+                const fa_view4* dout, const float* lse, const float* delta, const fa_view4* dk,
+                const fa_view4* dv, int B, int H, int Hk, int M, int N, int D, int causal,
+                float sm_scale, void* stream);
+int fa_bwd_dq(int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v,
+              const fa_view4* dout, const float* lse, const float* delta, const fa_view4* dq, int B,
+              int H, int Hk, int M, int N, int D, int causal, float sm_scale, void* stream);
+
+/* ------------------------------------------------------------------------- total attention --
+ * Replaces `_total_attention_kernel` (src/flag_attn/total.py:50-142; launches flash.py:128-140 and
+ * total.py:35-46): total[b,h,n] = sum_m softmax(scores)[m,n], recomputed from q, k and lse. */
+int fa_total_attn(int dtype, const fa_view4* q, const fa_view4* k, const float* lse, float* total,
+                  int B, int H, int Hk, int M, int N, int D, int causal, float sm_scale,
+                  void* stream);
+
+/* ----------------------------------------------------------- split-KV forward (flash decoding) --
+ * fa_splitkv_fwd     <- `_fwd_split_kv_kernel` (src/flag_attn/split_kv.py:14-160; launches
+ *                       flash.py:97-111, split_kv.py:298-312).
+ * fa_splitkv_combine <- `_fwd_combine_kv_splits` (split_kv.py:162-227; launches flash.py:113-125,
+ *                       split_kv.py:317-329).
+ * Split s covers keys [s * split_size, min(N, (s + 1) * split_size)).  part_o (B, H, S, M, D)
+ * contiguous, always fp16 as in the reference (flash.py:96); part_lse (B, H, S, M) fp32.  A split
+ * that holds no visible key for a row writes part_o = 0, part_lse = -inf. */
+int fa_splitkv_fwd(int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v, void* part_o,
+                   float* part_lse, int B, int H, int Hk, int M, int N, int D, int causal,
+                   float sm_scale, int num_splits, int split_size, void* stream);
+int fa_splitkv_combine(int dtype, const void* part_o, const float* part_lse, const fa_view4* o,
+                       float* lse, int B, int H, int M, int D, int num_splits, void* stream);
+
+/* ------------------------------------------------------------------------ piecewise attention --
+ * pw_fwd      <- piecewise `_fwd_kernel`    (src/flag_attn/piecewise.py:223-370, launch :50-69)
+ * pw_bwd_dkdv <- piecewise `_bwd_kv_kernel` (piecewise.py:450-627, launch :114-139)
+ * pw_bwd_dq   <- piecewise `_bwd_q_kernel`  (piecewise.py:630-792, launch :141-164)
+ * The score of (m, n) is q2.k2 when m + N - M - n >= dist_threshold, else q1.k1.  No grouped heads.
+ * The preprocess is fa_bwd_delta (piecewise.py:407-447 is the same computation). */
+int pw_fwd(int dtype, const fa_view4* q1, const fa_view4* k1, const fa_view4* q2, const fa_view4* k2,
+           const fa_view4* v, const fa_view4* o, float* lse, int B, int H, int M, int N, int D,
+           int dist_threshold, int causal, float sm_scale, void* stream);
+int pw_bwd_dkdv(int dtype, const fa_view4* q1, const fa_view4* k1, const fa_view4* q2,
+                const fa_view4* k2, const fa_view4* v, const fa_view4* dout, const float* lse,
+                const float* delta, const fa_view4* dk1, const fa_view4* dk2, const fa_view4* dv,
+                int B, int H, int M, int N, int D, int dist_threshold, int causal, float sm_scale,
+                void* stream);
+int pw_bwd_dq(int dtype, const fa_view4* q1, const fa_view4* k1, const fa_view4* q2,
+              const fa_view4* k2, const fa_view4* v, const fa_view4* dout, const float* lse,
+              const float* delta, const fa_view4* dq1, const fa_view4* dq2, int B, int H, int M,
+              int N, int D, int dist_threshold, int causal, float sm_scale, void* stream);
+
+/* ---------------------------------------------------------------------------- paged attention --
+ * paged_attn   <- `_paged_attn_kernel` (src/flag_attn/paged.py:204-349; launches :57-88, :112-142)
+ * paged_reduce <- `_paged_attn_v2_reduce_kernel` (paged.py:352-435; launch :144-162)
+ *
+ * query (num_seqs, Hq, D) with element strides q_stride_s, q_stride_h; key_cache / value_cache
+ * (num_blocks, Hkv, block_size, D) sharing the element strides kv_stride_{blk,h,tok};
+ * context_lens int32; block_tables int32 or int64 (bt_is_int64) with row stride bt_stride.
+ * partition_size == 0: one pass, `out` (num_seqs, Hq, D) with strides o_stride_s, o_stride_h.
+ * partition_size > 0 (a multiple of block_size): grid over num_parts partitions; writes
+ * tmp_out (num_seqs, Hkv, num_parts, G, D) in the cache dtype and max_logits / exp_sums
+ * (num_seqs, Hkv, num_parts, G) fp32, to be merged by paged_reduce. */
+int paged_attn(int dtype, void* out, int64_t o_stride_s, int64_t o_stride_h, const void* query,
+               int64_t q_stride_s, int64_t q_stride_h, const void* key_cache, const void* value_cache,
+               int64_t kv_stride_blk, int64_t kv_stride_h, int64_t kv_stride_tok,
+               const int32_t* context_lens, const void* block_tables, int bt_is_int64,
+               int64_t bt_stride, float attn_scale, int num_seqs, int num_q_heads, int num_kv_heads,
+               int head_size, int block_size, int partition_size, int num_parts, void* tmp_out,
+               float* max_logits, float* exp_sums, void* stream);
+int paged_reduce(int dtype, void* out, int64_t o_stride_s, int64_t o_stride_h, const void* tmp_out,
+                 const float* max_logits, const float* exp_sums, const int32_t* context_lens,
+                 int num_seqs, int num_q_heads, int num_kv_heads, int head_size, int partition_size,
+                 int num_parts, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLAGATTN_H */

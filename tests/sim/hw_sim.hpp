@@ -1,0 +1,249 @@
+// Host stand-in for csrc/hw.hpp: runs a HIP kernel body lane by lane on the CPU.
+//
+// TEST INFRASTRUCTURE.  Each lane of a workgroup is a ucontext fiber; a wavefront's 64 fibers are
+// run in turn up to their next collective operation (matrix multiply, transposing LDS read, lane
+// exchange, workgroup barrier), the operation is evaluated for the whole wavefront with the operand
+// layouts measured on gfx950, and the fibers resume.  LDS is a heap block of exactly the requested
+// size, so AddressSanitizer sees every out-of-range LDS or global access a kernel would make.
+#pragma once
+#include <stdint.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#include <math.h>
+#include <ucontext.h>
+#include <functional>
+#include <vector>
+
+#if defined(__has_feature)
+#if __has_feature(address_sanitizer)
+#define HWSIM_ASAN 1
+extern "C" void __sanitizer_start_switch_fiber(void** fake_stack_save, const void* bottom, size_t size);
+extern "C" void __sanitizer_finish_switch_fiber(void* fake_stack_save, const void** bottom_old, size_t* size_old);
+#endif
+#endif
+
+typedef void* hipStream_t;
+struct dim3 { unsigned x, y, z; dim3(unsigned a = 1, unsigned b = 1, unsigned c = 1) : x(a), y(b), z(c) {} };
+
+namespace hwsim {
+
+enum Op { OP_NONE, OP_DONE, OP_BARRIER, OP_MFMA32, OP_MFMA16, OP_TR, OP_SHFL };
+
+struct Lane {
+  ucontext_t ctx;
+  char* stack = nullptr;
+  Op op = OP_NONE;
+  float a[8], b[8], c[16], out[16];
+  const void* addr = nullptr;
+  uint16_t tr[4];
+  float sh_in = 0, sh_out = 0;
+  int mask = 0;
+  void* fake = nullptr;
+};
+
+constexpr size_t kStack = 256 * 1024;
+inline std::vector<Lane> lanes;
+inline int cur = 0;
+inline ucontext_t sched_ctx;
+inline void* sched_fake = nullptr;
+inline const void* sched_bottom = nullptr;
+inline size_t sched_size = 0;
+inline int bx, by, bz, gx;
+inline unsigned char* lds = nullptr;
+inline std::function<void()> body;
+
+inline void to_sched() {
+#ifdef HWSIM_ASAN
+  __sanitizer_start_switch_fiber(&lanes[cur].fake, sched_bottom, sched_size);
+#endif
+  swapcontext(&lanes[cur].ctx, &sched_ctx);
+#ifdef HWSIM_ASAN
+  __sanitizer_finish_switch_fiber(lanes[cur].fake, &sched_bottom, &sched_size);
+#endif
+}
+inline void yield(Op op) { lanes[cur].op = op; to_sched(); }
+
+inline void entry() {
+#ifdef HWSIM_ASAN
+  __sanitizer_finish_switch_fiber(nullptr, &sched_bottom, &sched_size);
+#endif
+  body();
+  lanes[cur].op = OP_DONE;
+#ifdef HWSIM_ASAN
+  __sanitizer_start_switch_fiber(nullptr, sched_bottom, sched_size);
+#endif
+  swapcontext(&lanes[cur].ctx, &sched_ctx);
+}
+
+inline void resume(int l) {
+  cur = l;
+#ifdef HWSIM_ASAN
+  __sanitizer_start_switch_fiber(&sched_fake, lanes[l].stack, kStack);
+#endif
+  swapcontext(&sched_ctx, &lanes[l].ctx);
+#ifdef HWSIM_ASAN
+  __sanitizer_finish_switch_fiber(sched_fake, nullptr, nullptr);
+#endif
+}
+
+inline void die(const char* msg) { fprintf(stderr, "hwsim: %s\n", msg); abort(); }
+
+inline void eval_wave(int base, Op op) {
+  Lane* L = &lanes[base];
+  if (op == OP_MFMA32) {
+    for (int i = 0; i < 32; ++i)
+      for (int j = 0; j < 32; ++j) {
+        int h = (i % 8) / 4, r = 4 * (i / 8) + i % 4;
+        float s = L[h * 32 + j].c[r];
+        for (int k = 0; k < 16; ++k) s += L[(k / 8) * 32 + i].a[k % 8] * L[(k / 8) * 32 + j].b[k % 8];
+        L[h * 32 + j].out[r] = s;
+      }
+  } else if (op == OP_MFMA16) {
+    for (int i = 0; i < 16; ++i)
+      for (int j = 0; j < 16; ++j) {
+        int q = i / 4, r = i % 4;
+        float s = L[q * 16 + j].c[r];
+        for (int k = 0; k < 32; ++k) s += L[(k / 8) * 16 + i].a[k % 8] * L[(k / 8) * 16 + j].b[k % 8];
+        L[q * 16 + j].out[r] = s;
+      }
+  } else if (op == OP_TR) {
+    for (int l = 0; l < 64; ++l) {
+      int g = l / 16, i = l % 16;
+      for (int e = 0; e < 4; ++e) {
+        const uint16_t* src = (const uint16_t*)L[g * 16 + 4 * e + i / 4].addr;
+        L[l].tr[e] = src[i % 4];
+      }
+    }
+  } else if (op == OP_SHFL) {
+    for (int l = 0; l < 64; ++l) L[l].sh_out = L[l ^ L[l].mask].sh_in;
+  }
+}
+
+// Runs `fn` once per lane of every workgroup of the grid, one workgroup at a time.
+inline void run_grid(dim3 grid, int threads, size_t lds_bytes, std::function<void()> fn) {
+  if (threads % 64) die("workgroup size must be a multiple of the wavefront size");
+  body = fn;
+  gx = (int)grid.x;
+  lanes.resize(threads);
+  for (auto& ln : lanes)
+    if (!ln.stack) ln.stack = (char*)malloc(kStack);
+  int waves = threads / 64;
+  std::vector<int> state(waves);  // 0 running, 1 at barrier, 2 done
+  for (unsigned z = 0; z < grid.z; ++z)
+    for (unsigned y = 0; y < grid.y; ++y)
+      for (unsigned x = 0; x < grid.x; ++x) {
+        bx = (int)x; by = (int)y; bz = (int)z;
+        lds = (unsigned char*)malloc(lds_bytes ? lds_bytes : 1);
+        memset(lds, 0xA5, lds_bytes);
+        for (int t = 0; t < threads; ++t) {
+          getcontext(&lanes[t].ctx);
+          lanes[t].ctx.uc_stack.ss_sp = lanes[t].stack;
+          lanes[t].ctx.uc_stack.ss_size = kStack;
+          lanes[t].ctx.uc_link = nullptr;
+          lanes[t].op = OP_NONE;
+          makecontext(&lanes[t].ctx, (void (*)())entry, 0);
+        }
+        for (auto& s : state) s = 0;
+        for (;;) {
+          int done = 0, waiting = 0;
+          for (int w = 0; w < waves; ++w) {
+            if (state[w] == 2) { ++done; continue; }
+            if (state[w] == 1) { ++waiting; continue; }
+            for (int l = 0; l < 64; ++l) resume(w * 64 + l);
+            Op op = lanes[w * 64].op;
+            for (int l = 1; l < 64; ++l)
+              if (lanes[w * 64 + l].op != op) die("lanes of one wavefront reached different collective operations");
+            if (op == OP_DONE) { state[w] = 2; ++done; }
+            else if (op == OP_BARRIER) { state[w] = 1; ++waiting; }
+            else eval_wave(w * 64, op);
+          }
+          if (done == waves) break;
+          if (done + waiting == waves) {
+            if (done) die("workgroup barrier reached by some wavefronts after others exited");
+            for (auto& s : state) s = 0;
+          }
+        }
+        free(lds);
+        lds = nullptr;
+      }
+}
+
+}  // namespace hwsim
+
+namespace hw {
+
+using half_t = _Float16;
+using bf16_t = __bf16;
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef short short8v __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+#define FA_DEVICE inline
+#define FA_KERNEL
+#define FA_LAUNCH_BOUNDS(n)
+#define FA_LDS_DECL(name) unsigned char* name = ::hwsim::lds
+
+inline int thread_id() { return hwsim::cur; }
+inline int block_x() { return hwsim::bx; }
+inline int block_y() { return hwsim::by; }
+inline int block_z() { return hwsim::bz; }
+inline int grid_x() { return hwsim::gx; }
+inline void block_sync() { hwsim::yield(hwsim::OP_BARRIER); }
+
+template <class V8> inline f32x16 mfma32_any(V8 a, V8 b, f32x16 c) {
+  hwsim::Lane& ln = hwsim::lanes[hwsim::cur];
+  for (int e = 0; e < 8; ++e) { ln.a[e] = (float)a[e]; ln.b[e] = (float)b[e]; }
+  for (int r = 0; r < 16; ++r) ln.c[r] = c[r];
+  hwsim::yield(hwsim::OP_MFMA32);
+  hwsim::Lane& l2 = hwsim::lanes[hwsim::cur];
+  f32x16 d;
+  for (int r = 0; r < 16; ++r) d[r] = l2.out[r];
+  return d;
+}
+inline f32x16 mfma32(half8 a, half8 b, f32x16 c) { return mfma32_any(a, b, c); }
+inline f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) { return mfma32_any(a, b, c); }
+
+template <class V8> inline f32x4 mfma16_any(V8 a, V8 b, f32x4 c) {
+  hwsim::Lane& ln = hwsim::lanes[hwsim::cur];
+  for (int e = 0; e < 8; ++e) { ln.a[e] = (float)a[e]; ln.b[e] = (float)b[e]; }
+  for (int r = 0; r < 4; ++r) ln.c[r] = c[r];
+  hwsim::yield(hwsim::OP_MFMA16);
+  hwsim::Lane& l2 = hwsim::lanes[hwsim::cur];
+  f32x4 d;
+  for (int r = 0; r < 4; ++r) d[r] = l2.out[r];
+  return d;
+}
+inline f32x4 mfma16(half8 a, half8 b, f32x4 c) { return mfma16_any(a, b, c); }
+inline f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) { return mfma16_any(a, b, c); }
+
+inline short4v lds_read_tr16(const void* p) {
+  hwsim::lanes[hwsim::cur].addr = p;
+  // touch the 8 bytes here so the sanitizer attributes a bad address to the lane that passed it
+  volatile uint16_t probe = ((const uint16_t*)p)[0] ^ ((const uint16_t*)p)[3];
+  (void)probe;
+  hwsim::yield(hwsim::OP_TR);
+  hwsim::Lane& ln = hwsim::lanes[hwsim::cur];
+  short4v r;
+  for (int e = 0; e < 4; ++e) r[e] = (short)ln.tr[e];
+  return r;
+}
+
+inline float shfl_xor(float x, int mask) {
+  hwsim::Lane& ln = hwsim::lanes[hwsim::cur];
+  ln.sh_in = x;
+  ln.mask = mask;
+  hwsim::yield(hwsim::OP_SHFL);
+  return hwsim::lanes[hwsim::cur].sh_out;
+}
+inline float xor32(float x) { return shfl_xor(x, 32); }
+
+inline float exp2_fast(float x) { return exp2f(x); }
+inline float log_nat(float x) { return logf(x); }
+
+}  // namespace hw
