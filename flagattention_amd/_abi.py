@@ -55,13 +55,16 @@ def check(code, what):
     raise KernelError(f"{what}: HIP error {code}")
 
 
+def is_kernel_ready(t):
+    return (t.stride(-1) == 1 and t.data_ptr() % 16 == 0
+            and all(_stride(t, d) % 8 == 0 for d in range(t.dim() - 1)))
+
+
 def kernel_ready(t):
     """The kernels move 16 bytes at a time: unit inner stride, 16-byte aligned base, strides that are
     multiples of 8 elements.  Anything else is copied (the reference copies when the inner stride is
     not 1, src/flag_attn/flash.py:14-17)."""
-    ok = (t.stride(-1) == 1 and t.data_ptr() % 16 == 0
-          and all(_stride(t, d) % 8 == 0 for d in range(t.dim() - 1)))
-    return t if ok else t.clone(memory_format=torch.contiguous_format)
+    return t if is_kernel_ready(t) else t.clone(memory_format=torch.contiguous_format)
 
 
 def fa_fwd(lib, q, k, v, o, lse, causal, sm_scale):
@@ -77,3 +80,84 @@ def pw_fwd(lib, q1, k1, q2, k2, v, o, lse, w, causal, sm_scale):
     check(lib.pw_fwd(dtype_code(q1), view4(q1), view4(k1), view4(q2), view4(k2), view4(v), view4(o),
                      ptr(lse), B, H, M, N, D, int(w), int(causal), float(sm_scale), stream_of(q1)),
           "pw_fwd")
+
+
+def fa_bwd_delta(lib, o, do, delta):
+    B, H, M, D = o.shape
+    check(lib.fa_bwd_delta(dtype_code(o), view4(o), view4(do), ptr(delta), B, H, M, D, stream_of(o)),
+          "fa_bwd_delta")
+
+
+def fa_bwd_dkdv(lib, q, k, v, do, lse, delta, dk, dv, causal, sm_scale):
+    B, H, M, D = q.shape
+    Hk, N = k.shape[1], k.shape[2]
+    check(lib.fa_bwd_dkdv(dtype_code(q), view4(q), view4(k), view4(v), view4(do), ptr(lse), ptr(delta),
+                          view4(dk), view4(dv), B, H, Hk, M, N, D, int(causal), float(sm_scale),
+                          stream_of(q)), "fa_bwd_dkdv")
+
+
+def fa_bwd_dq(lib, q, k, v, do, lse, delta, dq, causal, sm_scale):
+    B, H, M, D = q.shape
+    Hk, N = k.shape[1], k.shape[2]
+    check(lib.fa_bwd_dq(dtype_code(q), view4(q), view4(k), view4(v), view4(do), ptr(lse), ptr(delta),
+                        view4(dq), B, H, Hk, M, N, D, int(causal), float(sm_scale), stream_of(q)),
+          "fa_bwd_dq")
+
+
+def pw_bwd_dkdv(lib, q1, k1, q2, k2, v, do, lse, delta, dk1, dk2, dv, w, causal, sm_scale):
+    B, H, M, D = q1.shape
+    N = k1.shape[2]
+    check(lib.pw_bwd_dkdv(dtype_code(q1), view4(q1), view4(k1), view4(q2), view4(k2), view4(v), view4(do),
+                          ptr(lse), ptr(delta), view4(dk1), view4(dk2), view4(dv), B, H, M, N, D,
+                          int(w), int(causal), float(sm_scale), stream_of(q1)), "pw_bwd_dkdv")
+
+
+def pw_bwd_dq(lib, q1, k1, q2, k2, v, do, lse, delta, dq1, dq2, w, causal, sm_scale):
+    B, H, M, D = q1.shape
+    N = k1.shape[2]
+    check(lib.pw_bwd_dq(dtype_code(q1), view4(q1), view4(k1), view4(q2), view4(k2), view4(v), view4(do),
+                        ptr(lse), ptr(delta), view4(dq1), view4(dq2), B, H, M, N, D, int(w),
+                        int(causal), float(sm_scale), stream_of(q1)), "pw_bwd_dq")
+
+
+def fa_total_attn(lib, q, k, lse, total, causal, sm_scale):
+    B, H, M, D = q.shape
+    Hk, N = k.shape[1], k.shape[2]
+    check(lib.fa_total_attn(dtype_code(q), view4(q), view4(k), ptr(lse), ptr(total), B, H, Hk, M, N, D,
+                            int(causal), float(sm_scale), stream_of(q)), "fa_total_attn")
+
+
+def fa_splitkv_fwd(lib, q, k, v, part_o, part_lse, causal, sm_scale, num_splits, split_size):
+    B, H, M, D = q.shape
+    Hk, N = k.shape[1], k.shape[2]
+    check(lib.fa_splitkv_fwd(dtype_code(q), view4(q), view4(k), view4(v), ptr(part_o), ptr(part_lse),
+                             B, H, Hk, M, N, D, int(causal), float(sm_scale), int(num_splits),
+                             int(split_size), stream_of(q)), "fa_splitkv_fwd")
+
+
+def fa_splitkv_combine(lib, part_o, part_lse, o, lse, num_splits):
+    B, H, M, D = o.shape
+    check(lib.fa_splitkv_combine(dtype_code(o), ptr(part_o), ptr(part_lse), view4(o), ptr(lse),
+                                 B, H, M, D, int(num_splits), stream_of(o)), "fa_splitkv_combine")
+
+
+def paged_attn(lib, out, query, key_cache, value_cache, context_lens, block_tables, scale,
+               partition_size, num_parts, tmp_out, max_logits, exp_sums):
+    num_seqs, Hq, D = query.shape
+    _, Hkv, block_size, _ = key_cache.shape
+    assert block_tables.dtype in (torch.int32, torch.int64)
+    check(lib.paged_attn(dtype_code(query), ptr(out), out.stride(0), out.stride(1),
+                         ptr(query), query.stride(0), query.stride(1),
+                         ptr(key_cache), ptr(value_cache),
+                         key_cache.stride(0), key_cache.stride(1), key_cache.stride(2),
+                         ptr(context_lens), ptr(block_tables), int(block_tables.dtype == torch.int64),
+                         block_tables.stride(0), float(scale), num_seqs, Hq, Hkv, D, block_size,
+                         int(partition_size), int(num_parts), ptr(tmp_out), ptr(max_logits),
+                         ptr(exp_sums), stream_of(query)), "paged_attn")
+
+
+def paged_reduce(lib, out, tmp_out, max_logits, exp_sums, context_lens, Hkv, partition_size, num_parts):
+    num_seqs, Hq, D = out.shape
+    check(lib.paged_reduce(dtype_code(out), ptr(out), out.stride(0), out.stride(1), ptr(tmp_out),
+                           ptr(max_logits), ptr(exp_sums), ptr(context_lens), num_seqs, Hq, Hkv, D,
+                           int(partition_size), int(num_parts), stream_of(out)), "paged_reduce")

@@ -73,4 +73,174 @@ int pw_fwd(int dtype, const fa_view4* q1, const fa_view4* k1, const fa_view4* q2
   return fa::run_fwd(p, true, (hipStream_t)stream);
 }
 
+int fa_bwd_delta(int dtype, const fa_view4* o, const fa_view4* dout, float* delta, int B, int H,
+                 int M, int D, void* stream) {
+  if (!view_ok(o) || !view_ok(dout) || !delta) return FA_ERR_BAD_ARGUMENT;
+  if (!head_dim_ok(D)) return FA_ERR_UNSUPPORTED;
+  fa::BwdParams p = {};
+  p.o = to_view(o); p.dout = to_view(dout); p.delta = delta;
+  p.B = B; p.H = H; p.M = M; p.D = D; p.dtype = dtype;
+  return fa::run_bwd_delta(p, (hipStream_t)stream);
+}
+
+static int fill_bwd(fa::BwdParams& p, int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v,
+                    const fa_view4* dout, const float* lse, const float* delta, int B, int H, int Hk,
+                    int M, int N, int D, int causal, float sm_scale) {
+  if (!view_ok(q) || !view_ok(k) || !view_ok(v) || !view_ok(dout) || !lse || !delta)
+    return FA_ERR_BAD_ARGUMENT;
+  if (!head_dim_ok(D)) return FA_ERR_UNSUPPORTED;
+  if (Hk <= 0 || H % Hk) return FA_ERR_BAD_ARGUMENT;
+  p.q = to_view(q); p.k = to_view(k); p.v = to_view(v); p.dout = to_view(dout);
+  p.lse = lse; p.delta = const_cast<float*>(delta);
+  p.B = B; p.H = H; p.M = M; p.N = N; p.D = D;
+  p.group = H / Hk; p.causal = causal; p.sm_scale = sm_scale; p.dtype = dtype;
+  return 0;
+}
+
+int fa_bwd_dkdv(int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v,
+                const fa_view4* dout, const float* lse, const float* delta, const fa_view4* dk,
+                const fa_view4* dv, int B, int H, int Hk, int M, int N, int D, int causal,
+                float sm_scale, void* stream) {
+  fa::BwdParams p = {};
+  int rc = fill_bwd(p, dtype, q, k, v, dout, lse, delta, B, H, Hk, M, N, D, causal, sm_scale);
+  if (rc) return rc;
+  if (!view_ok(dk) || !view_ok(dv)) return FA_ERR_BAD_ARGUMENT;
+  p.dk = to_view(dk); p.dv = to_view(dv);
+  return fa::run_bwd_dkdv(p, false, (hipStream_t)stream);
+}
+
+int fa_bwd_dq(int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v,
+              const fa_view4* dout, const float* lse, const float* delta, const fa_view4* dq, int B,
+              int H, int Hk, int M, int N, int D, int causal, float sm_scale, void* stream) {
+  fa::BwdParams p = {};
+  int rc = fill_bwd(p, dtype, q, k, v, dout, lse, delta, B, H, Hk, M, N, D, causal, sm_scale);
+  if (rc) return rc;
+  if (!view_ok(dq)) return FA_ERR_BAD_ARGUMENT;
+  p.dq = to_view(dq);
+  return fa::run_bwd_dq(p, false, (hipStream_t)stream);
+}
+
+int pw_bwd_dkdv(int dtype, const fa_view4* q1, const fa_view4* k1, const fa_view4* q2,
+                const fa_view4* k2, const fa_view4* v, const fa_view4* dout, const float* lse,
+                const float* delta, const fa_view4* dk1, const fa_view4* dk2, const fa_view4* dv,
+                int B, int H, int M, int N, int D, int dist_threshold, int causal, float sm_scale,
+                void* stream) {
+  fa::BwdParams p = {};
+  int rc = fill_bwd(p, dtype, q1, k1, v, dout, lse, delta, B, H, H, M, N, D, causal, sm_scale);
+  if (rc) return rc;
+  if (!view_ok(q2) || !view_ok(k2) || !view_ok(dk1) || !view_ok(dk2) || !view_ok(dv))
+    return FA_ERR_BAD_ARGUMENT;
+  p.q2 = to_view(q2); p.k2 = to_view(k2);
+  p.dk = to_view(dk1); p.dk2 = to_view(dk2); p.dv = to_view(dv);
+  p.w = dist_threshold;
+  return fa::run_bwd_dkdv(p, true, (hipStream_t)stream);
+}
+
+int pw_bwd_dq(int dtype, const fa_view4* q1, const fa_view4* k1, const fa_view4* q2,
+              const fa_view4* k2, const fa_view4* v, const fa_view4* dout, const float* lse,
+              const float* delta, const fa_view4* dq1, const fa_view4* dq2, int B, int H, int M,
+              int N, int D, int dist_threshold, int causal, float sm_scale, void* stream) {
+  fa::BwdParams p = {};
+  int rc = fill_bwd(p, dtype, q1, k1, v, dout, lse, delta, B, H, H, M, N, D, causal, sm_scale);
+  if (rc) return rc;
+  if (!view_ok(q2) || !view_ok(k2) || !view_ok(dq1) || !view_ok(dq2)) return FA_ERR_BAD_ARGUMENT;
+  p.q2 = to_view(q2); p.k2 = to_view(k2);
+  p.dq = to_view(dq1); p.dq2 = to_view(dq2);
+  p.w = dist_threshold;
+  return fa::run_bwd_dq(p, true, (hipStream_t)stream);
+}
+
+int fa_total_attn(int dtype, const fa_view4* q, const fa_view4* k, const float* lse, float* total,
+                  int B, int H, int Hk, int M, int N, int D, int causal, float sm_scale,
+                  void* stream) {
+  if (!view_ok(q) || !view_ok(k) || !lse || !total) return FA_ERR_BAD_ARGUMENT;
+  if (!head_dim_ok(D)) return FA_ERR_UNSUPPORTED;
+  if (Hk <= 0 || H % Hk) return FA_ERR_BAD_ARGUMENT;
+  fa::TotalParams p = {};
+  p.q = to_view(q); p.k = to_view(k); p.lse = lse; p.total = total;
+  p.B = B; p.H = H; p.M = M; p.N = N; p.D = D;
+  p.group = H / Hk; p.causal = causal; p.sm_scale = sm_scale; p.dtype = dtype;
+  return fa::run_total(p, (hipStream_t)stream);
+}
+
+int fa_splitkv_fwd(int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v, void* part_o,
+                   float* part_lse, int B, int H, int Hk, int M, int N, int D, int causal,
+                   float sm_scale, int num_splits, int split_size, void* stream) {
+  if (!view_ok(q) || !view_ok(k) || !view_ok(v) || !part_o || !part_lse) return FA_ERR_BAD_ARGUMENT;
+  if (((uintptr_t)part_o) & 15) return FA_ERR_BAD_ARGUMENT;
+  if (!head_dim_ok(D)) return FA_ERR_UNSUPPORTED;
+  if (Hk <= 0 || H % Hk) return FA_ERR_BAD_ARGUMENT;
+  fa::SplitParams p = {};
+  p.q = to_view(q); p.k = to_view(k); p.v = to_view(v);
+  p.part_o = part_o; p.part_lse = part_lse;
+  p.B = B; p.H = H; p.M = M; p.N = N; p.D = D;
+  p.group = H / Hk; p.causal = causal;
+  p.num_splits = num_splits; p.split_size = split_size;
+  p.sm_scale = sm_scale; p.dtype = dtype;
+  return fa::run_splitkv(p, (hipStream_t)stream);
+}
+
+int fa_splitkv_combine(int dtype, const void* part_o, const float* part_lse, const fa_view4* o,
+                       float* lse, int B, int H, int M, int D, int num_splits, void* stream) {
+  if (!part_o || !part_lse || !view_ok(o) || !lse) return FA_ERR_BAD_ARGUMENT;
+  if (((uintptr_t)part_o) & 15) return FA_ERR_BAD_ARGUMENT;
+  if (!head_dim_ok(D)) return FA_ERR_UNSUPPORTED;
+  fa::CombineParams p = {};
+  p.part_o = part_o; p.part_lse = part_lse; p.o = to_view(o); p.lse = lse;
+  p.B = B; p.H = H; p.M = M; p.D = D; p.num_splits = num_splits; p.dtype = dtype;
+  return fa::run_combine(p, (hipStream_t)stream);
+}
+
+static int fill_paged(fa::PagedParams& p, int dtype, void* out, int64_t o_stride_s, int64_t o_stride_h,
+                      const int32_t* context_lens, int num_seqs, int num_q_heads, int num_kv_heads,
+                      int head_size, int partition_size, int num_parts, void* tmp_out, float* max_logits,
+                      float* exp_sums) {
+  if (!out || !context_lens) return FA_ERR_BAD_ARGUMENT;
+  if (partition_size > 0 && (!tmp_out || !max_logits || !exp_sums)) return FA_ERR_BAD_ARGUMENT;
+  p.out = out; p.o_ss = o_stride_s; p.o_sh = o_stride_h;
+  p.context_lens = context_lens;
+  p.num_seqs = num_seqs; p.Hq = num_q_heads; p.Hkv = num_kv_heads; p.D = head_size;
+  p.partition_size = partition_size; p.num_parts = num_parts;
+  p.tmp_out = tmp_out; p.max_logits = max_logits; p.exp_sums = exp_sums;
+  p.dtype = dtype;
+  return 0;
+}
+
+int paged_attn(int dtype, void* out, int64_t o_stride_s, int64_t o_stride_h, const void* query,
+               int64_t q_stride_s, int64_t q_stride_h, const void* key_cache, const void* value_cache,
+               int64_t kv_stride_blk, int64_t kv_stride_h, int64_t kv_stride_tok,
+               const int32_t* context_lens, const void* block_tables, int bt_is_int64,
+               int64_t bt_stride, float attn_scale, int num_seqs, int num_q_heads, int num_kv_heads,
+               int head_size, int block_size, int partition_size, int num_parts, void* tmp_out,
+               float* max_logits, float* exp_sums, void* stream) {
+  fa::PagedParams p = {};
+  int rc = fill_paged(p, dtype, out, o_stride_s, o_stride_h, context_lens, num_seqs, num_q_heads,
+                      num_kv_heads, head_size, partition_size, num_parts, tmp_out, max_logits, exp_sums);
+  if (rc) return rc;
+  if (!query || !key_cache || !value_cache || !block_tables) return FA_ERR_BAD_ARGUMENT;
+  if ((((uintptr_t)query) | ((uintptr_t)key_cache) | ((uintptr_t)value_cache)) & 15) return FA_ERR_BAD_ARGUMENT;
+  if ((q_stride_s | q_stride_h | kv_stride_blk | kv_stride_h | kv_stride_tok) % 8) return FA_ERR_BAD_ARGUMENT;
+  if (!(head_size == 16 || head_size == 32 || head_size == 64 || head_size == 128 || head_size == 256))
+    return FA_ERR_UNSUPPORTED;
+  p.q = query; p.q_ss = q_stride_s; p.q_sh = q_stride_h;
+  p.kc = key_cache; p.vc = value_cache;
+  p.kv_sblk = kv_stride_blk; p.kv_sh = kv_stride_h; p.kv_stok = kv_stride_tok;
+  p.block_tables = block_tables; p.bt64 = bt_is_int64; p.bt_stride = bt_stride;
+  p.scale = attn_scale; p.block_size = block_size;
+  return fa::run_paged(p, (hipStream_t)stream);
+}
+
+int paged_reduce(int dtype, void* out, int64_t o_stride_s, int64_t o_stride_h, const void* tmp_out,
+                 const float* max_logits, const float* exp_sums, const int32_t* context_lens,
+                 int num_seqs, int num_q_heads, int num_kv_heads, int head_size, int partition_size,
+                 int num_parts, void* stream) {
+  fa::PagedParams p = {};
+  int rc = fill_paged(p, dtype, out, o_stride_s, o_stride_h, context_lens, num_seqs, num_q_heads,
+                      num_kv_heads, head_size, partition_size, num_parts, const_cast<void*>(tmp_out),
+                      const_cast<float*>(max_logits), const_cast<float*>(exp_sums));
+  if (rc) return rc;
+  p.block_size = 1;
+  return fa::run_paged_reduce(p, (hipStream_t)stream);
+}
+
 }  // extern "C"

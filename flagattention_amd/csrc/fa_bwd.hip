@@ -1,0 +1,511 @@
+// FlashAttention-2 backward for gfx950 (and the piecewise variant): the row-dot preprocess, a
+// kernel that owns a block of keys and produces dK/dV, and a kernel that owns a block of queries and
+// produces dQ.  As in the reference there is no atomic read-modify-write: every output tile has
+// exactly one writer.
+//
+// Replaces `_bwd_preprocess` (src/flag_attn/flash.py:522-568), `_bwd_kv_kernel` (flash.py:571-745),
+// `_bwd_q_kernel` (flash.py:748-909) and their piecewise counterparts
+// (src/flag_attn/piecewise.py:407-447, 450-627, 630-792).
+//
+// Shared scheme: P is recomputed as exp2(S * scale * log2e - L * log2e) from the saved
+// log-normalizer; masked entries are removed by select (never by multiplying), because a row that
+// saw no key has L = -inf and would give inf * 0.
+//
+//  dK/dV kernel: a wavefront owns 32 keys; K and V rows sit in registers as B operands of
+//    S = Q K^T and dP = dO V^T (queries x keys, one key per lane).  P and dS then come out of the MFMA
+//    in the A-operand layout of dV += P^T dO and dK += dS^T Q, whose B operands (dO, Q with the
+//    query index as contraction index) are fetched from the LDS tiles with the transposing read.
+//  dQ kernel: a wavefront owns 32 queries; Q and dO rows sit in registers as B operands of
+//    S^T = K Q^T and dP^T = V dO^T (keys x queries, one query per lane, so L and delta are per-lane
+//    scalars); dS^T is the B operand of dQ^T += K^T dS^T, with K^T read transposed from LDS.
+#include "common.hpp"
+#include "params.hpp"
+
+namespace fa {
+
+// ------------------------------------------------------------------------------ preprocess ----
+template <class T, int D>
+FA_KERNEL void FA_LAUNCH_BOUNDS(kThreads) fa_bwd_delta_kernel(BwdParams p) {
+  constexpr int kLanesPerRow = D / 8;
+  constexpr int kRows = kThreads / kLanesPerRow;
+  const int tid = hw::thread_id();
+  const int row = hw::block_x() * kRows + tid / kLanesPerRow;
+  const int col = (tid % kLanesPerRow) * 8;
+  const int head = hw::block_y(), batch = hw::block_z();
+  float acc = 0.f;
+  if (row < p.M) {
+    const T* o = (const T*)p.o.ptr + batch * p.o.sb + head * p.o.sh + (int64_t)row * p.o.st + col;
+    const T* g = (const T*)p.dout.ptr + batch * p.dout.sb + head * p.dout.sh + (int64_t)row * p.dout.st + col;
+    auto ov = hw::as_v8<T>(*(const u32x4*)o);
+    auto gv = hw::as_v8<T>(*(const u32x4*)g);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc += (float)ov[e] * (float)gv[e];
+  }
+#pragma unroll
+  for (int s = 1; s < kLanesPerRow; s <<= 1) acc += hw::shfl_xor(acc, s);
+  if (row < p.M && (tid % kLanesPerRow) == 0)
+    p.delta[((int64_t)batch * p.H + head) * p.M + row] = acc;
+}
+
+template <class T>
+static int launch_delta(const BwdParams& p, hipStream_t stream) {
+  auto rows = [](int D) { return kThreads / (D / 8); };
+  switch (p.D) {
+    case 16: return launch(fa_bwd_delta_kernel<T, 16>, dim3((p.M + rows(16) - 1) / rows(16), p.H, p.B), 0, stream, p);
+    case 32: return launch(fa_bwd_delta_kernel<T, 32>, dim3((p.M + rows(32) - 1) / rows(32), p.H, p.B), 0, stream, p);
+    case 64: return launch(fa_bwd_delta_kernel<T, 64>, dim3((p.M + rows(64) - 1) / rows(64), p.H, p.B), 0, stream, p);
+    case 128: return launch(fa_bwd_delta_kernel<T, 128>, dim3((p.M + rows(128) - 1) / rows(128), p.H, p.B), 0, stream, p);
+  }
+  return kUnsupported;
+}
+
+int run_bwd_delta(const BwdParams& p, hipStream_t stream) {
+  if (p.B <= 0 || p.H <= 0 || p.M <= 0) return kBadArgument;
+  if (p.dtype == kDtypeF16) return launch_delta<hw::half_t>(p, stream);
+  if (p.dtype == kDtypeBF16) return launch_delta<hw::bf16_t>(p, stream);
+  return kUnsupported;
+}
+
+// ------------------------------------------------------------------------------- dK and dV ----
+template <class T, int D, bool PW>
+struct KvCfg {
+  static constexpr int BN = 128;  // keys per workgroup (32 per wavefront)
+  static constexpr int BM = 64;   // queries per pipeline step
+  static constexpr int DV = D < 32 ? 32 : D;
+  static constexpr int KSTEPS = D / 16;
+  static constexpr int LD = DV + 8;
+  static constexpr int TILE = BM * LD;
+  static constexpr int NTILES = PW ? 3 : 2;  // Q, (Q2), dO
+  static constexpr size_t STAGE_BYTES = NTILES * TILE * sizeof(T) + 2 * BM * sizeof(float);
+  static constexpr size_t LDS_BYTES = 2 * STAGE_BYTES;
+};
+
+template <class T, int D, bool PW>
+FA_KERNEL void FA_LAUNCH_BOUNDS(kThreads) fa_bwd_dkdv_kernel(BwdParams p) {
+  using C = KvCfg<T, D, PW>;
+  using V8 = typename hw::Elem<T>::v8;
+  FA_LDS_DECL(smem);
+
+  const int tid = hw::thread_id(), lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, hh = lane >> 5;
+  const int head = hw::block_y(), batch = hw::block_z();
+  const int hk = head / p.group;
+  const int M = p.M, N = p.N, pseq = N - M;
+  const int n0 = hw::block_x() * C::BN, nw = n0 + wave * 32, my_n = nw + l32;
+
+  const T* qb = (const T*)p.q.ptr + batch * p.q.sb + head * p.q.sh;
+  const T* q2b = PW ? (const T*)p.q2.ptr + batch * p.q2.sb + head * p.q2.sh : nullptr;
+  const T* gb = (const T*)p.dout.ptr + batch * p.dout.sb + head * p.dout.sh;
+  const T* kb = (const T*)p.k.ptr + batch * p.k.sb + hk * p.k.sh;
+  const T* k2b = PW ? (const T*)p.k2.ptr + batch * p.k2.sb + hk * p.k2.sh : nullptr;
+  const T* vb = (const T*)p.v.ptr + batch * p.v.sb + hk * p.v.sh;
+  const float* lse = p.lse + ((int64_t)batch * p.H + head) * M;
+  const float* dlt = p.delta + ((int64_t)batch * p.H + head) * M;
+
+  // K, (K2), V rows of this lane as B operands (k = 16 kk + 8 hh + 0..7)
+  V8 kreg[C::KSTEPS], vreg[C::KSTEPS], k2reg[PW ? C::KSTEPS : 1];
+#pragma unroll
+  for (int kk = 0; kk < C::KSTEPS; ++kk) {
+    u32x4 a = {0u, 0u, 0u, 0u}, b = a, c = a;
+    if (my_n < N) {
+      a = *(const u32x4*)(kb + (int64_t)my_n * p.k.st + 16 * kk + 8 * hh);
+      b = *(const u32x4*)(vb + (int64_t)my_n * p.v.st + 16 * kk + 8 * hh);
+      if (PW) c = *(const u32x4*)(k2b + (int64_t)my_n * p.k2.st + 16 * kk + 8 * hh);
+    }
+    kreg[kk] = hw::as_v8<T>(a);
+    vreg[kk] = hw::as_v8<T>(b);
+    if (PW) k2reg[kk] = hw::as_v8<T>(c);
+  }
+
+  // first query tile that can see a key of this block under the causal mask
+  int m_lo = 0;
+  if (p.causal) m_lo = (imax(0, n0 - pseq) / C::BM) * C::BM;
+  const int n_tiles = m_lo < M ? cdiv(M - m_lo, C::BM) : 0;
+
+  if (C::DV != D) {
+    T* z = (T*)smem;
+    for (int i = tid; i < (int)(C::LDS_BYTES / sizeof(T)); i += kThreads) z[i] = (T)0.f;
+    hw::block_sync();
+  }
+
+  f32x16 dk[C::DV / 32], dv[C::DV / 32], dk2[PW ? C::DV / 32 : 1];
+#pragma unroll
+  for (int i = 0; i < C::DV / 32; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { dk[i][r] = 0.f; dv[i][r] = 0.f; if (PW) dk2[i][r] = 0.f; }
+
+  auto tile_needs_near = [&](int m0) { return !PW || (m0 + pseq - (n0 + C::BN - 1) < p.w); };
+  auto tile_needs_far = [&](int m0) { return PW && (m0 + C::BM - 1 + pseq - n0 >= p.w); };
+
+  TileRegs<C::BM, D> qr, q2r, gr;
+  float l_reg = 0.f, d_reg = 0.f;
+  auto fetch = [&](int m0) {
+    if (tile_needs_near(m0)) tile_fetch<T, C::BM, D>(qr, qb, p.q.st, m0, M, tid);
+    if (tile_needs_far(m0)) tile_fetch<T, C::BM, D>(q2r, q2b, p.q2.st, m0, M, tid);
+    tile_fetch<T, C::BM, D>(gr, gb, p.dout.st, m0, M, tid);
+    if (tid < C::BM) {
+      int m = m0 + tid;
+      // rows past M get L = +inf, hence P = 0
+      l_reg = m < M ? lse[m] * kLog2e : __builtin_inff();
+      d_reg = m < M ? dlt[m] : 0.f;
+    }
+  };
+  auto commit = [&](int m0, int stage) {
+    unsigned char* base = smem + stage * C::STAGE_BYTES;
+    T* s = (T*)base;
+    if (tile_needs_near(m0)) tile_commit<T, C::BM, D, C::LD>(qr, s, tid);
+    if (tile_needs_far(m0)) tile_commit<T, C::BM, D, C::LD>(q2r, s + C::TILE, tid);
+    tile_commit<T, C::BM, D, C::LD>(gr, s + (C::NTILES - 1) * C::TILE, tid);
+    float* f = (float*)(base + C::NTILES * C::TILE * sizeof(T));
+    if (tid < C::BM) { f[tid] = l_reg; f[C::BM + tid] = d_reg; }
+  };
+
+  if (n_tiles > 0) { fetch(m_lo); commit(m_lo, 0); }
+  hw::block_sync();
+
+  const float c2 = p.sm_scale * kLog2e;
+
+  for (int it = 0; it < n_tiles; ++it) {
+    const int m0 = m_lo + it * C::BM;
+    const bool more = it + 1 < n_tiles;
+    if (more) fetch(m0 + C::BM);
+
+    const unsigned char* base = smem + (it & 1) * C::STAGE_BYTES;
+    const T* sQ = (const T*)base;
+    const T* sQ2 = sQ + C::TILE;
+    const T* sG = sQ + (C::NTILES - 1) * C::TILE;
+    const float* sL = (const float*)(base + C::NTILES * C::TILE * sizeof(T));
+    const float* sDl = sL + C::BM;
+
+#pragma unroll
+    for (int sb = 0; sb < C::BM / 32; ++sb) {
+      const int mr0 = m0 + sb * 32;
+      // every (m, n) of this 32 x 32 block is masked: nothing to add
+      if (p.causal && (mr0 + 31 + pseq < nw)) continue;
+      bool near = true, far = false;
+      if (PW) {
+        near = (mr0 + pseq - (nw + 31)) < p.w;
+        far = (mr0 + 31 + pseq - nw) >= p.w;
+      }
+      f32x16 s, s2, dp;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { s[r] = 0.f; s2[r] = 0.f; dp[r] = 0.f; }
+      if (near) {
+#pragma unroll
+        for (int kk = 0; kk < C::KSTEPS; ++kk)
+          s = hw::mfma32(operand_rowmajor<T, C::LD>(sQ, sb * 32, 16 * kk, lane), kreg[kk], s);
+      }
+      if (PW && far) {
+#pragma unroll
+        for (int kk = 0; kk < C::KSTEPS; ++kk)
+          s2 = hw::mfma32(operand_rowmajor<T, C::LD>(sQ2, sb * 32, 16 * kk, lane), k2reg[kk], s2);
+      }
+#pragma unroll
+      for (int kk = 0; kk < C::KSTEPS; ++kk)
+        dp = hw::mfma32(operand_rowmajor<T, C::LD>(sG, sb * 32, 16 * kk, lane), vreg[kk], dp);
+
+      const bool need_mask = p.causal && (mr0 + pseq < nw + 31);
+      f32x16 pr, ds, ds2;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int ml = sb * 32 + block_row(r, hh);
+        const int m = m0 + ml;
+        float sv = s[r];
+        bool is_far = false;
+        if (PW) {
+          is_far = (m + pseq - my_n) >= p.w;
+          sv = is_far ? s2[r] : s[r];
+        }
+        float pv = hw::exp2_fast(fmaf(sv, c2, -sL[ml]));
+        if (need_mask) pv = (m + pseq >= my_n) ? pv : 0.f;
+        float dsv = pv * (dp[r] - sDl[ml]);
+        pr[r] = pv;
+        if (PW) {
+          ds[r] = is_far ? 0.f : dsv;
+          ds2[r] = is_far ? dsv : 0.f;
+        } else {
+          ds[r] = dsv;
+        }
+      }
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        V8 pa = pack_half_block<T>(pr, c);
+#pragma unroll
+        for (int db = 0; db < C::DV / 32; ++db)
+          dv[db] = hw::mfma32(pa, operand_transposed<T, C::LD>(sG, sb * 32 + 16 * c, db * 32, lane), dv[db]);
+        if (near) {
+          V8 da = pack_half_block<T>(ds, c);
+#pragma unroll
+          for (int db = 0; db < C::DV / 32; ++db)
+            dk[db] = hw::mfma32(da, operand_transposed<T, C::LD>(sQ, sb * 32 + 16 * c, db * 32, lane), dk[db]);
+        }
+        if (PW && far) {
+          V8 da2 = pack_half_block<T>(ds2, c);
+#pragma unroll
+          for (int db = 0; db < C::DV / 32; ++db)
+            dk2[db] = hw::mfma32(da2, operand_transposed<T, C::LD>(sQ2, sb * 32 + 16 * c, db * 32, lane), dk2[db]);
+        }
+      }
+    }
+
+    if (more) commit(m0 + C::BM, (it + 1) & 1);
+    hw::block_sync();
+  }
+
+  // ---- store: result block (keys x D) has D along lanes, keys along registers ----
+  T* dkb = (T*)p.dk.ptr + batch * p.dk.sb + head * p.dk.sh;
+  T* dvb = (T*)p.dv.ptr + batch * p.dv.sb + head * p.dv.sh;
+  T* dk2b = PW ? (T*)p.dk2.ptr + batch * p.dk2.sb + head * p.dk2.sh : nullptr;
+#pragma unroll
+  for (int db = 0; db < C::DV / 32; ++db) {
+    const int d = db * 32 + l32;
+    if (d < D) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int n = nw + block_row(r, hh);
+        if (n < N) {
+          dkb[(int64_t)n * p.dk.st + d] = (T)(dk[db][r] * p.sm_scale);
+          dvb[(int64_t)n * p.dv.st + d] = (T)dv[db][r];
+          if (PW) dk2b[(int64_t)n * p.dk2.st + d] = (T)(dk2[db][r] * p.sm_scale);
+        }
+      }
+    }
+  }
+}
+
+// ----------------------------------------------------------------------------------- dQ ----
+template <class T, int D, bool PW>
+struct QCfg {
+  static constexpr int BM = 128;  // queries per workgroup (32 per wavefront)
+  static constexpr int BN = 64;   // keys per pipeline step
+  static constexpr int DV = D < 32 ? 32 : D;
+  static constexpr int KSTEPS = D / 16;
+  static constexpr int LD = DV + 8;
+  static constexpr int TILE = BN * LD;
+  static constexpr int NTILES = PW ? 3 : 2;  // K, (K2), V
+  static constexpr size_t STAGE_BYTES = NTILES * TILE * sizeof(T);
+  static constexpr size_t LDS_BYTES = 2 * STAGE_BYTES;
+};
+
+template <class T, int D, bool PW>
+FA_KERNEL void FA_LAUNCH_BOUNDS(kThreads) fa_bwd_dq_kernel(BwdParams p) {
+  using C = QCfg<T, D, PW>;
+  using V8 = typename hw::Elem<T>::v8;
+  FA_LDS_DECL(smem);
+  T* lds = (T*)smem;
+
+  const int tid = hw::thread_id(), lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, hh = lane >> 5;
+  const int mb = hw::grid_x() - 1 - hw::block_x();
+  const int head = hw::block_y(), batch = hw::block_z();
+  const int hk = head / p.group;
+  const int M = p.M, N = p.N, pseq = N - M;
+  const int m0 = mb * C::BM, mw = m0 + wave * 32, my_m = mw + l32;
+
+  const T* qb = (const T*)p.q.ptr + batch * p.q.sb + head * p.q.sh;
+  const T* q2b = PW ? (const T*)p.q2.ptr + batch * p.q2.sb + head * p.q2.sh : nullptr;
+  const T* gb = (const T*)p.dout.ptr + batch * p.dout.sb + head * p.dout.sh;
+  const T* kb = (const T*)p.k.ptr + batch * p.k.sb + hk * p.k.sh;
+  const T* k2b = PW ? (const T*)p.k2.ptr + batch * p.k2.sb + hk * p.k2.sh : nullptr;
+  const T* vb = (const T*)p.v.ptr + batch * p.v.sb + hk * p.v.sh;
+
+  V8 qreg[C::KSTEPS], greg[C::KSTEPS], q2reg[PW ? C::KSTEPS : 1];
+#pragma unroll
+  for (int kk = 0; kk < C::KSTEPS; ++kk) {
+    u32x4 a = {0u, 0u, 0u, 0u}, b = a, c = a;
+    if (my_m < M) {
+      a = *(const u32x4*)(qb + (int64_t)my_m * p.q.st + 16 * kk + 8 * hh);
+      b = *(const u32x4*)(gb + (int64_t)my_m * p.dout.st + 16 * kk + 8 * hh);
+      if (PW) c = *(const u32x4*)(q2b + (int64_t)my_m * p.q2.st + 16 * kk + 8 * hh);
+    }
+    qreg[kk] = hw::as_v8<T>(a);
+    greg[kk] = hw::as_v8<T>(b);
+    if (PW) q2reg[kk] = hw::as_v8<T>(c);
+  }
+  // rows past M get L = +inf, hence P = 0
+  const int64_t row_off = ((int64_t)batch * p.H + head) * M + my_m;
+  const float l_row = my_m < M ? p.lse[row_off] * kLog2e : __builtin_inff();
+  const float d_row = my_m < M ? p.delta[row_off] : 0.f;
+
+  int hi = N;
+  if (p.causal) hi = imin(N, pseq + m0 + C::BM);
+  const int n_tiles = hi > 0 ? cdiv(hi, C::BN) : 0;
+
+  if (C::DV != D) {
+    for (int i = tid; i < (int)(C::LDS_BYTES / sizeof(T)); i += kThreads) lds[i] = (T)0.f;
+    hw::block_sync();
+  }
+
+  f32x16 dq[C::DV / 32], dq2[PW ? C::DV / 32 : 1];
+#pragma unroll
+  for (int i = 0; i < C::DV / 32; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { dq[i][r] = 0.f; if (PW) dq2[i][r] = 0.f; }
+
+  auto tile_needs_near = [&](int n0) { return !PW || (m0 + pseq - (n0 + C::BN - 1) < p.w); };
+  auto tile_needs_far = [&](int n0) { return PW && (m0 + C::BM - 1 + pseq - n0 >= p.w); };
+
+  TileRegs<C::BN, D> kr, k2r, vr;
+  auto fetch = [&](int n0) {
+    if (tile_needs_near(n0)) tile_fetch<T, C::BN, D>(kr, kb, p.k.st, n0, N, tid);
+    if (tile_needs_far(n0)) tile_fetch<T, C::BN, D>(k2r, k2b, p.k2.st, n0, N, tid);
+    tile_fetch<T, C::BN, D>(vr, vb, p.v.st, n0, N, tid);
+  };
+  auto commit = [&](int n0, int stage) {
+    T* s = (T*)(smem + stage * C::STAGE_BYTES);
+    if (tile_needs_near(n0)) tile_commit<T, C::BN, D, C::LD>(kr, s, tid);
+    if (tile_needs_far(n0)) tile_commit<T, C::BN, D, C::LD>(k2r, s + C::TILE, tid);
+    tile_commit<T, C::BN, D, C::LD>(vr, s + (C::NTILES - 1) * C::TILE, tid);
+  };
+
+  if (n_tiles > 0) { fetch(0); commit(0, 0); }
+  hw::block_sync();
+
+  const float c2 = p.sm_scale * kLog2e;
+
+  for (int it = 0; it < n_tiles; ++it) {
+    const int n0 = it * C::BN;
+    const bool more = it + 1 < n_tiles;
+    if (more) fetch(n0 + C::BN);
+
+    const T* sK = (const T*)(smem + (it & 1) * C::STAGE_BYTES);
+    const T* sK2 = sK + C::TILE;
+    const T* sV = sK + (C::NTILES - 1) * C::TILE;
+
+#pragma unroll
+    for (int nb = 0; nb < C::BN / 32; ++nb) {
+      const int nlo = n0 + nb * 32;
+      if (p.causal && (mw + 31 + pseq < nlo)) continue;  // block fully masked for this wavefront
+      bool near = true, far = false;
+      if (PW) {
+        near = (mw + pseq - (nlo + 31)) < p.w;
+        far = (mw + 31 + pseq - nlo) >= p.w;
+      }
+      f32x16 s, s2, dp;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { s[r] = 0.f; s2[r] = 0.f; dp[r] = 0.f; }
+      if (near) {
+#pragma unroll
+        for (int kk = 0; kk < C::KSTEPS; ++kk)
+          s = hw::mfma32(operand_rowmajor<T, C::LD>(sK, nb * 32, 16 * kk, lane), qreg[kk], s);
+      }
+      if (PW && far) {
+#pragma unroll
+        for (int kk = 0; kk < C::KSTEPS; ++kk)
+          s2 = hw::mfma32(operand_rowmajor<T, C::LD>(sK2, nb * 32, 16 * kk, lane), q2reg[kk], s2);
+      }
+#pragma unroll
+      for (int kk = 0; kk < C::KSTEPS; ++kk)
+        dp = hw::mfma32(operand_rowmajor<T, C::LD>(sV, nb * 32, 16 * kk, lane), greg[kk], dp);
+
+      const bool need_mask = (nlo + 32 > N) || (p.causal && (nlo + 31 > pseq + mw));
+      f32x16 ds, ds2;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int n = nlo + block_row(r, hh);
+        float sv = s[r];
+        bool is_far = false;
+        if (PW) {
+          is_far = (my_m + pseq - n) >= p.w;
+          sv = is_far ? s2[r] : s[r];
+        }
+        float pv = hw::exp2_fast(fmaf(sv, c2, -l_row));
+        if (need_mask) pv = ((n < N) && (!p.causal || (my_m + pseq >= n))) ? pv : 0.f;
+        float dsv = pv * (dp[r] - d_row);
+        if (PW) {
+          ds[r] = is_far ? 0.f : dsv;
+          ds2[r] = is_far ? dsv : 0.f;
+        } else {
+          ds[r] = dsv;
+        }
+      }
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        if (near) {
+          V8 db_ = pack_half_block<T>(ds, c);
+#pragma unroll
+          for (int db = 0; db < C::DV / 32; ++db)
+            dq[db] = hw::mfma32(operand_transposed<T, C::LD>(sK, nb * 32 + 16 * c, db * 32, lane), db_, dq[db]);
+        }
+        if (PW && far) {
+          V8 db2 = pack_half_block<T>(ds2, c);
+#pragma unroll
+          for (int db = 0; db < C::DV / 32; ++db)
+            dq2[db] = hw::mfma32(operand_transposed<T, C::LD>(sK2, nb * 32 + 16 * c, db * 32, lane), db2, dq2[db]);
+        }
+      }
+    }
+
+    if (more) commit(n0 + C::BN, (it + 1) & 1);
+    hw::block_sync();
+  }
+
+  // ---- store dQ^T blocks: lane owns one query row, registers run along D ----
+  if (my_m < M) {
+    T* o1 = (T*)p.dq.ptr + batch * p.dq.sb + head * p.dq.sh + (int64_t)my_m * p.dq.st;
+    T* o2 = PW ? (T*)p.dq2.ptr + batch * p.dq2.sb + head * p.dq2.sh + (int64_t)my_m * p.dq2.st : nullptr;
+#pragma unroll
+    for (int db = 0; db < C::DV / 32; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        int d = db * 32 + 8 * g + 4 * hh;
+        if (d < D) {
+          hw::u32x2 w;
+          w[0] = (uint32_t)hw::bits16<T>(dq[db][4 * g + 0] * p.sm_scale) | ((uint32_t)hw::bits16<T>(dq[db][4 * g + 1] * p.sm_scale) << 16);
+          w[1] = (uint32_t)hw::bits16<T>(dq[db][4 * g + 2] * p.sm_scale) | ((uint32_t)hw::bits16<T>(dq[db][4 * g + 3] * p.sm_scale) << 16);
+          *(hw::u32x2*)(o1 + d) = w;
+          if (PW) {
+            hw::u32x2 w2;
+            w2[0] = (uint32_t)hw::bits16<T>(dq2[db][4 * g + 0] * p.sm_scale) | ((uint32_t)hw::bits16<T>(dq2[db][4 * g + 1] * p.sm_scale) << 16);
+            w2[1] = (uint32_t)hw::bits16<T>(dq2[db][4 * g + 2] * p.sm_scale) | ((uint32_t)hw::bits16<T>(dq2[db][4 * g + 3] * p.sm_scale) << 16);
+            *(hw::u32x2*)(o2 + d) = w2;
+          }
+        }
+      }
+  }
+}
+
+// ------------------------------------------------------------------------------ launchers ----
+template <class T, bool PW>
+static int launch_dkdv(const BwdParams& p, hipStream_t stream) {
+  dim3 grid((p.N + 127) / 128, p.H, p.B);
+  switch (p.D) {
+    case 16: return launch(fa_bwd_dkdv_kernel<T, 16, PW>, grid, KvCfg<T, 16, PW>::LDS_BYTES, stream, p);
+    case 32: return launch(fa_bwd_dkdv_kernel<T, 32, PW>, grid, KvCfg<T, 32, PW>::LDS_BYTES, stream, p);
+    case 64: return launch(fa_bwd_dkdv_kernel<T, 64, PW>, grid, KvCfg<T, 64, PW>::LDS_BYTES, stream, p);
+    case 128: return launch(fa_bwd_dkdv_kernel<T, 128, PW>, grid, KvCfg<T, 128, PW>::LDS_BYTES, stream, p);
+  }
+  return kUnsupported;
+}
+
+template <class T, bool PW>
+static int launch_dq(const BwdParams& p, hipStream_t stream) {
+  dim3 grid((p.M + 127) / 128, p.H, p.B);
+  switch (p.D) {
+    case 16: return launch(fa_bwd_dq_kernel<T, 16, PW>, grid, QCfg<T, 16, PW>::LDS_BYTES, stream, p);
+    case 32: return launch(fa_bwd_dq_kernel<T, 32, PW>, grid, QCfg<T, 32, PW>::LDS_BYTES, stream, p);
+    case 64: return launch(fa_bwd_dq_kernel<T, 64, PW>, grid, QCfg<T, 64, PW>::LDS_BYTES, stream, p);
+    case 128: return launch(fa_bwd_dq_kernel<T, 128, PW>, grid, QCfg<T, 128, PW>::LDS_BYTES, stream, p);
+  }
+  return kUnsupported;
+}
+
+int run_bwd_dkdv(const BwdParams& p, bool piecewise, hipStream_t stream) {
+  if (p.B <= 0 || p.H <= 0 || p.M <= 0 || p.N <= 0 || p.group <= 0) return kBadArgument;
+  if (p.dtype == kDtypeF16)
+    return piecewise ? launch_dkdv<hw::half_t, true>(p, stream) : launch_dkdv<hw::half_t, false>(p, stream);
+  if (p.dtype == kDtypeBF16)
+    return piecewise ? launch_dkdv<hw::bf16_t, true>(p, stream) : launch_dkdv<hw::bf16_t, false>(p, stream);
+  return kUnsupported;
+}
+
+int run_bwd_dq(const BwdParams& p, bool piecewise, hipStream_t stream) {
+  if (p.B <= 0 || p.H <= 0 || p.M <= 0 || p.N <= 0 || p.group <= 0) return kBadArgument;
+  if (p.dtype == kDtypeF16)
+    return piecewise ? launch_dq<hw::half_t, true>(p, stream) : launch_dq<hw::half_t, false>(p, stream);
+  if (p.dtype == kDtypeBF16)
+    return piecewise ? launch_dq<hw::bf16_t, true>(p, stream) : launch_dq<hw::bf16_t, false>(p, stream);
+  return kUnsupported;
+}
+
+}  // namespace fa

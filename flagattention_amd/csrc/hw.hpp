@@ -41,6 +41,13 @@ FA_DEVICE int block_y() { return (int)blockIdx.y; }
 FA_DEVICE int block_z() { return (int)blockIdx.z; }
 FA_DEVICE int grid_x() { return (int)gridDim.x; }
 FA_DEVICE void block_sync() { __syncthreads(); }
+// Orders the LDS traffic of one wavefront: writes issued by any lane before the call are visible
+// to reads issued by any lane after it (LDS serves a wavefront's requests in order; this only stops
+// the compiler from moving accesses across).
+FA_DEVICE void wave_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+}
 
 // D(32x32) += A(32x16) * B(16x32).  Lane l holds, for h = l / 32:
 //   A[i = l % 32][k = 8h + e], e = 0..7          B[k = 8h + e][j = l % 32]

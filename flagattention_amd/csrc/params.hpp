@@ -62,3 +62,47 @@ int run_bwd_dkdv(const BwdParams& p, bool piecewise, hipStream_t stream);
 int run_bwd_dq(const BwdParams& p, bool piecewise, hipStream_t stream);
 int run_total(const TotalParams& p, hipStream_t stream);
 }  // namespace fa
+
+namespace fa {
+
+struct SplitParams {
+  View4 q, k, v;
+  void* part_o;      // (B, H, S, M, D) fp16, contiguous
+  float* part_lse;   // (B, H, S, M)
+  int B, H, M, N, D;
+  int group;
+  int causal;
+  int num_splits, split_size;
+  float sm_scale;
+  int dtype;
+};
+
+struct CombineParams {
+  const void* part_o;
+  const float* part_lse;
+  View4 o;
+  float* lse;  // (B, H, M)
+  int B, H, M, D, num_splits;
+  int dtype;
+};
+
+struct PagedParams {
+  void* out; int64_t o_ss, o_sh;          // final output (num_seqs, Hq, D) when partition_size == 0
+  const void* q; int64_t q_ss, q_sh;
+  const void* kc; const void* vc;
+  int64_t kv_sblk, kv_sh, kv_stok;
+  const int32_t* context_lens;
+  const void* block_tables; int bt64; int64_t bt_stride;
+  float scale;
+  int num_seqs, Hq, Hkv, D, block_size;
+  int partition_size, num_parts;
+  void* tmp_out; float* max_logits; float* exp_sums;
+  int dtype;
+};
+
+int run_splitkv(const SplitParams& p, hipStream_t stream);
+int run_combine(const CombineParams& p, hipStream_t stream);
+int run_paged(const PagedParams& p, hipStream_t stream);
+int run_paged_reduce(const PagedParams& p, hipStream_t stream);
+
+}  // namespace fa

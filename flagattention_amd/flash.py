@@ -1,0 +1,116 @@
+"""``flash_attention``: FlashAttention-2 forward/backward on gfx950 HIP kernels.
+
+Host-side counterpart of ``src/flag_attn/flash.py:23-286`` of the reference: same signature, same
+return convention, same autograd contract (``save_for_backward(q, k, v, o, L)``, gradients for
+q, k, v only, gradients flowing into the auxiliary outputs are ignored).  The Triton launches are
+replaced by calls into the C-ABI kernel library.
+"""
+import math
+
+import torch
+
+from . import _abi, _lib
+from .split_kv import num_splits_heuristic, split_kv_forward, SPLIT_BLOCK_M, SPLIT_BLOCK_N
+from .total import _total_attention
+
+__all__ = ["attention"]
+
+_HEAD_DIMS = (16, 32, 64, 128)
+
+
+def get_fwd_config(B, H, M, N, D, causal):
+    """(BLOCK_M, BLOCK_N, num_stages, num_warps) of the dense forward kernel.
+
+    Kept as an overridable module-level hook like ``src/flag_attn/flash.py:290-322``; on gfx950 the
+    tile shape is compiled into the kernel (128 query rows per workgroup, 64-key pipeline stages,
+    two LDS stages, four 64-lane wavefronts), so the value is informational."""
+    return (128, 64, 2, 4)
+
+
+def get_bwd_config(B, H, M, N, D, causal):
+    """(BLOCK_M, BLOCK_N, num_stages, num_warps) of the dK/dV kernel (``flash.py:493-519`` hook)."""
+    return (64, 128, 2, 4)
+
+
+class FlashAttention(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, causal, sm_scale, dropout_p, return_log_normalizer,
+                return_total_attention, return_seed_offset):
+        Dq, Dk, Dv = q.shape[-1], k.shape[-1], v.shape[-1]
+        assert Dq == Dk == Dv, "feature size of q, k, v should be equal"
+        assert Dk in _HEAD_DIMS
+        B, H, M, D = q.shape
+        N = k.shape[2]
+        Hk, Hv = k.shape[1], v.shape[1]
+        assert Hk == Hv, "num of heads in k and v should be equal"
+        assert H % Hk == 0, "number of heads in q must be a multiple of that in k & v"
+        if dropout_p > 0:
+            raise NotImplementedError("dropout is not implemented by the gfx950 kernels yet")
+        if sm_scale is None:
+            sm_scale = 1.0 / math.sqrt(D)
+
+        lib = _lib.get()
+        q, k, v = _abi.kernel_ready(q), _abi.kernel_ready(k), _abi.kernel_ready(v)
+
+        with torch.cuda.device(q.device):
+            num_cus = lib.fa_num_cus()
+            splits = num_splits_heuristic(B, H, M, N, SPLIT_BLOCK_M, SPLIT_BLOCK_N, num_cus, 128)
+            if splits > 1:
+                o, L = split_kv_forward(lib, q, k, v, causal, sm_scale, splits)
+            else:
+                o = torch.empty_like(q)
+                if not _abi.is_kernel_ready(o):
+                    o = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+                L = torch.empty((B, H, M), device=q.device, dtype=torch.float32)
+                _abi.fa_fwd(lib, q, k, v, o, L, causal, sm_scale)
+            tot_attn = None
+            if return_total_attention:
+                tot_attn = _total_attention(lib, q, k, L, causal, sm_scale)
+
+        ctx.save_for_backward(q, k, v, o, L)
+        ctx.sm_scale = sm_scale
+        ctx.causal = causal
+
+        if return_log_normalizer or return_total_attention or return_seed_offset:
+            return (o,
+                    L if return_log_normalizer else None,
+                    tot_attn if return_total_attention else None,
+                    None, None)
+        return o
+
+    @staticmethod
+    def backward(ctx, do, *ignored):
+        q, k, v, o, L = ctx.saved_tensors
+        sm_scale, causal = ctx.sm_scale, ctx.causal
+        B, H, M, D = q.shape
+        N, Hk = k.shape[2], k.shape[1]
+        group = H // Hk
+        lib = _lib.get()
+        do = _abi.kernel_ready(do)
+        with torch.cuda.device(q.device):
+            delta = torch.empty_like(L)
+            _abi.fa_bwd_delta(lib, o, do, delta)
+            # one dK/dV slice per query head; groups are summed afterwards (as flash.py:205-206,250-251)
+            dk = torch.empty((B, H, N, D), dtype=k.dtype, device=q.device)
+            dv = torch.empty((B, H, N, D), dtype=v.dtype, device=q.device)
+            _abi.fa_bwd_dkdv(lib, q, k, v, do, L, delta, dk, dv, causal, sm_scale)
+            dq = torch.empty((B, H, M, D), dtype=q.dtype, device=q.device)
+            _abi.fa_bwd_dq(lib, q, k, v, do, L, delta, dq, causal, sm_scale)
+            if group > 1:
+                dk = dk.reshape(B, Hk, group, N, D).sum(2)
+                dv = dv.reshape(B, Hk, group, N, D).sum(2)
+        return dq, dk, dv, None, None, None, None, None, None
+
+
+def attention(q, k, v, causal=False, sm_scale=None, dropout_p=0.0,
+              return_log_normalizer=False, return_total_attention=False, return_seed_offset=False):
+    """FlashAttention-2.
+
+    q (batch, heads_q, seqlen_q, headdim); k, v (batch, heads_k, seqlen_k, headdim); heads_q must be
+    a multiple of heads_k.  ``causal`` masks with bottom-right alignment.  Returns ``out`` or, when
+    any ``return_*`` flag is set, ``(out, log_normalizer|None, total_attention|None, seed|None,
+    offset|None)`` -- exactly the reference's convention (``src/flag_attn/flash.py:150-160``).
+    ``dropout_p > 0`` raises ``NotImplementedError``.
+    """
+    return FlashAttention.apply(q, k, v, causal, sm_scale, dropout_p, return_log_normalizer,
+                                return_total_attention, return_seed_offset)

@@ -1,0 +1,83 @@
+"""``paged_attention``: single-token decode over a block-table-indexed key/value cache.
+
+Host-side counterpart of ``src/flag_attn/paged.py:6-163`` of the reference: same signature, same
+meaning of ``num_splits`` (0 = choose, 1 = one pass, > 1 = that many partitions of
+``next_power_of_2(ceil(max_context_len / num_splits))`` tokens), partitions merged by a reduce kernel.
+"""
+import torch
+
+from . import _abi, _lib
+
+__all__ = ["attention"]
+
+_HEAD_SIZES = (16, 32, 64, 128, 256)
+
+
+def _next_pow2(x):
+    return 1 << max(0, (int(x) - 1).bit_length())
+
+
+def choose_partitioning(num_seqs, num_kv_heads, block_size, max_context_len, num_cus):
+    """Automatic partitioning for ``num_splits == 0`` on a device with ``num_cus`` compute units.
+
+    One workgroup handles one (sequence, kv head, partition).  Partitions are cut so that the launch
+    has about four workgroups per compute unit when the batch alone cannot provide them, but never
+    shorter than 512 tokens (each wavefront then still streams four 32-key steps) and always a
+    multiple of the cache block size.  Returns (num_splits, partition_size); num_splits == 1 means a
+    single pass that writes the output directly."""
+    pairs = num_seqs * num_kv_heads
+    if max_context_len <= 1024 or pairs >= 8 * num_cus:
+        return 1, 0
+    want = max(1, -(-4 * num_cus // pairs))
+    size = max(512, _next_pow2(-(-max_context_len // want)))
+    size = -(-size // block_size) * block_size
+    splits = -(-max_context_len // size)
+    if splits <= 1:
+        return 1, 0
+    return splits, size
+
+
+def attention(query, key_cache, value_cache, context_lens, block_tables, attn_scale,
+              max_context_len, num_splits=0):
+    """query (num_seqs, heads_q, head_size); key_cache / value_cache (num_blocks, heads_kv, block_size,
+    head_size) with identical strides; context_lens (num_seqs,) int32; block_tables (num_seqs,
+    max_blocks_per_seq) int32 or int64.  Returns out shaped like ``query``."""
+    num_seqs, num_q_heads, head_size = query.shape
+    num_kv_heads, block_size = key_cache.shape[1], key_cache.shape[2]
+    assert key_cache.shape[3] == head_size and value_cache.shape == key_cache.shape
+    assert head_size in _HEAD_SIZES, f"head_size={head_size}"
+    assert num_q_heads % num_kv_heads == 0
+    assert key_cache.stride() == value_cache.stride(), "key and value cache must share their strides"
+    assert context_lens.dtype == torch.int32
+
+    lib = _lib.get()
+    if query.stride(-1) != 1 or query.data_ptr() % 16 or query.stride(0) % 8 or query.stride(1) % 8:
+        query = query.contiguous()
+    assert key_cache.stride(-1) == 1
+    context_lens = context_lens.contiguous()
+    if block_tables.stride(-1) != 1:
+        block_tables = block_tables.contiguous()
+    out = torch.empty(query.shape, dtype=query.dtype, device=query.device)
+    group = num_q_heads // num_kv_heads
+
+    with torch.cuda.device(query.device):
+        if num_splits == 0:
+            num_splits, partition_size = choose_partitioning(
+                num_seqs, num_kv_heads, block_size, max_context_len, lib.fa_num_cus())
+        elif num_splits > 1:
+            partition_size = _next_pow2(-(-max_context_len // num_splits))
+            assert partition_size >= block_size and partition_size % block_size == 0, \
+                f"partition_size={partition_size}, kv_block_size={block_size}"
+        if num_splits == 1:
+            _abi.paged_attn(lib, out, query, key_cache, value_cache, context_lens, block_tables,
+                            attn_scale, 0, 1, None, None, None)
+        else:
+            shape = (num_seqs, num_kv_heads, num_splits, group)
+            max_logits = torch.empty(shape, dtype=torch.float32, device=query.device)
+            exp_sums = torch.empty(shape, dtype=torch.float32, device=query.device)
+            tmp_out = torch.empty(shape + (head_size,), dtype=out.dtype, device=out.device)
+            _abi.paged_attn(lib, out, query, key_cache, value_cache, context_lens, block_tables,
+                            attn_scale, partition_size, num_splits, tmp_out, max_logits, exp_sums)
+            _abi.paged_reduce(lib, out, tmp_out, max_logits, exp_sums, context_lens, num_kv_heads,
+                              partition_size, num_splits)
+    return out

@@ -1,0 +1,71 @@
+"""``piecewise_attention``: attention whose score switches between two (q, k) pairs at a distance
+threshold, on gfx950 HIP kernels.
+
+Host-side counterpart of ``src/flag_attn/piecewise.py:25-191`` of the reference (same signature and
+autograd contract: five gradients, none for the threshold / flags).
+"""
+import math
+
+import torch
+
+from . import _abi, _lib
+
+__all__ = ["attention"]
+
+
+def get_fwd_config(B, H, M, N, D, causal):
+    """Informational; the tile shape is compiled into the kernel (``piecewise.py:194-221`` hook)."""
+    return (128, 64, 2, 4)
+
+
+def get_bwd_config(B, H, M, N, D, causal):
+    return (64, 128, 2, 4)
+
+
+class PiecewiseAttention(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q1, k1, q2, k2, v, w, causal, sm_scale):
+        Dq1, Dk1, Dq2, Dk2, Dv = (t.shape[-1] for t in (q1, k1, q2, k2, v))
+        assert Dq1 == Dk1 == Dq2 == Dk2 == Dv
+        assert Dk1 in (16, 32, 64, 128)
+        B, H, M, D = q1.shape
+        if sm_scale is None:
+            sm_scale = 1.0 / math.sqrt(D)
+        lib = _lib.get()
+        q1, k1, q2, k2, v = (_abi.kernel_ready(t) for t in (q1, k1, q2, k2, v))
+        with torch.cuda.device(q1.device):
+            o = torch.empty_like(q1)
+            if not _abi.is_kernel_ready(o):
+                o = torch.empty(q1.shape, dtype=q1.dtype, device=q1.device)
+            L = torch.empty((B, H, M), device=q1.device, dtype=torch.float32)
+            _abi.pw_fwd(lib, q1, k1, q2, k2, v, o, L, w, causal, sm_scale)
+        ctx.save_for_backward(q1, k1, q2, k2, v, o, L)
+        ctx.sm_scale, ctx.causal, ctx.w = sm_scale, causal, w
+        return o
+
+    @staticmethod
+    def backward(ctx, do):
+        q1, k1, q2, k2, v, o, L = ctx.saved_tensors
+        lib = _lib.get()
+        do = _abi.kernel_ready(do)
+        with torch.cuda.device(q1.device):
+            delta = torch.empty_like(L)
+            _abi.fa_bwd_delta(lib, o, do, delta)
+            dk1 = torch.empty(k1.shape, dtype=k1.dtype, device=k1.device)
+            dk2 = torch.empty(k2.shape, dtype=k2.dtype, device=k2.device)
+            dv = torch.empty(v.shape, dtype=v.dtype, device=v.device)
+            _abi.pw_bwd_dkdv(lib, q1, k1, q2, k2, v, do, L, delta, dk1, dk2, dv, ctx.w, ctx.causal, ctx.sm_scale)
+            dq1 = torch.empty(q1.shape, dtype=q1.dtype, device=q1.device)
+            dq2 = torch.empty(q2.shape, dtype=q2.dtype, device=q2.device)
+            _abi.pw_bwd_dq(lib, q1, k1, q2, k2, v, do, L, delta, dq1, dq2, ctx.w, ctx.causal, ctx.sm_scale)
+        return dq1, dk1, dq2, dk2, dv, None, None, None
+
+
+def attention(q1, k1, q2, k2, v, dist_threshold, causal=False, sm_scale=None):
+    """Piecewise attention.
+
+    q1, q2 (batch, heads, seqlen_q, headdim); k1, k2, v (batch, heads, seqlen_k, headdim).  The score
+    of query m and key n is ``q2[m].k2[n]`` when the signed distance ``m + seqlen_k - seqlen_q - n``
+    is at least ``dist_threshold`` and ``q1[m].k1[n]`` otherwise.  Returns out (batch, heads,
+    seqlen_q, headdim)."""
+    return PiecewiseAttention.apply(q1, k1, q2, k2, v, dist_threshold, causal, sm_scale)

@@ -1,0 +1,97 @@
+"""Split-KV forward (flash decoding): ``flash_attention_split_kv`` and the split-count rule.
+
+Host-side counterpart of ``src/flag_attn/split_kv.py:229-330`` of the reference.  The split kernel
+serves all query heads of a kv head from one workgroup, in steps of 32 keys per wavefront; the
+reference's (BLOCK_M, BLOCK_N) = (16, 128) only survives as the unit in which the split rule counts
+work, so that a given problem is split into the same number of pieces as in the reference.
+"""
+import math
+
+import torch
+
+from . import _abi, _lib
+
+__all__ = ["attention"]
+
+SPLIT_BLOCK_M, SPLIT_BLOCK_N = 16, 128
+
+
+def get_fwd_config(B, H, M, N, D, causal):
+    """Informational (``split_kv.py:229-231`` hook): (BLOCK_M, BLOCK_N, num_stages, num_warps)."""
+    return (SPLIT_BLOCK_M, SPLIT_BLOCK_N, 1, 4)
+
+
+def num_splits_heuristic(B, H, M, N, block_m, block_n, num_cus, max_splits):
+    """How many pieces to cut the key axis into (``split_kv.py:234-262``).
+
+    No split when the un-split grid already fills 80 % of the compute units.  Otherwise every split
+    count that does not leave a piece empty is scored by how full its last wave of workgroups is
+    (waves / ceil(waves)), and the smallest count within 85 % of the best score wins.
+    """
+    base_blocks = B * H * -(-M // block_m)
+    if base_blocks >= 0.8 * num_cus:
+        return 1
+    n_blocks = -(-N // block_n)
+    limit = min(num_cus, n_blocks, max_splits)
+    scored = []
+    for s in range(1, limit + 1):
+        per_split = -(-n_blocks // s)
+        if s > 1 and per_split * s - n_blocks >= per_split:
+            continue  # the last piece would be empty
+        waves = base_blocks * s / num_cus
+        scored.append((s, waves / math.ceil(waves)))
+    best = max((eff for _, eff in scored), default=0.0)
+    for s, eff in scored:
+        if eff >= 0.85 * best:
+            return s
+    return 1
+
+
+# spelling used by the reference, kept for callers that import it
+num_splits_herustic = num_splits_heuristic
+
+
+def _split_size(N, splits):
+    return -(-(-(-N // SPLIT_BLOCK_N)) // splits) * SPLIT_BLOCK_N
+
+
+def split_kv_forward(lib, q, k, v, causal, sm_scale, splits, combine=True):
+    """Runs the split kernel (+ merge).  Returns (o, L), or the fp16 partials when not merging."""
+    B, H, M, D = q.shape
+    N = k.shape[2]
+    part_lse = torch.empty((B, H, splits, M), dtype=torch.float32, device=q.device)
+    part_o = torch.empty((B, H, splits, M, D), dtype=torch.float16, device=q.device)
+    _abi.fa_splitkv_fwd(lib, q, k, v, part_o, part_lse, causal, sm_scale, splits, _split_size(N, splits))
+    if not combine:
+        return part_o, part_lse
+    L = torch.empty((B, H, M), dtype=torch.float32, device=q.device)
+    o = torch.empty_like(q)
+    if not _abi.is_kernel_ready(o):
+        o = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    _abi.fa_splitkv_combine(lib, part_o, part_lse, o, L, splits)
+    return o, L
+
+
+def attention(q, k, v, causal=False, sm_scale=None):
+    """Forward-only attention that always goes through the split-KV kernel (``split_kv.py:266-330``).
+
+    With a single split the fp16 partial output is returned directly, as the reference does."""
+    Dq, Dk, Dv = q.shape[-1], k.shape[-1], v.shape[-1]
+    assert Dq == Dk == Dv
+    assert Dk in (16, 32, 64, 128)
+    B, H, M, D = q.shape
+    N = k.shape[2]
+    Hk, Hv = k.shape[1], v.shape[1]
+    assert Hk == Hv, "num of heads in k and v should be equal"
+    assert H % Hk == 0, "number of heads in q must be a multiple of that in k & v"
+    if sm_scale is None:
+        sm_scale = 1.0 / math.sqrt(D)
+    lib = _lib.get()
+    q, k, v = _abi.kernel_ready(q), _abi.kernel_ready(k), _abi.kernel_ready(v)
+    with torch.cuda.device(q.device):
+        splits = num_splits_heuristic(B, H, M, N, SPLIT_BLOCK_M, SPLIT_BLOCK_N, lib.fa_num_cus(), 128)
+        if splits == 1:
+            part_o, _ = split_kv_forward(lib, q, k, v, causal, sm_scale, 1, combine=False)
+            return part_o.squeeze(2)
+        o, _ = split_kv_forward(lib, q, k, v, causal, sm_scale, splits)
+    return o

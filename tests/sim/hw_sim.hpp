@@ -28,7 +28,7 @@ struct dim3 { unsigned x, y, z; dim3(unsigned a = 1, unsigned b = 1, unsigned c 
 
 namespace hwsim {
 
-enum Op { OP_NONE, OP_DONE, OP_BARRIER, OP_MFMA32, OP_MFMA16, OP_TR, OP_SHFL };
+enum Op { OP_NONE, OP_DONE, OP_BARRIER, OP_MFMA32, OP_MFMA16, OP_TR, OP_SHFL, OP_WAVESYNC };
 
 struct Lane {
   ucontext_t ctx;
@@ -195,6 +195,7 @@ inline int block_y() { return hwsim::by; }
 inline int block_z() { return hwsim::bz; }
 inline int grid_x() { return hwsim::gx; }
 inline void block_sync() { hwsim::yield(hwsim::OP_BARRIER); }
+inline void wave_sync() { hwsim::yield(hwsim::OP_WAVESYNC); }
 
 template <class V8> inline f32x16 mfma32_any(V8 a, V8 b, f32x16 c) {
   hwsim::Lane& ln = hwsim::lanes[hwsim::cur];

@@ -1,0 +1,164 @@
+"""GPU parity tests of flash_attention (forward, split-KV path, backward, auxiliary outputs).
+
+Shapes, scales and layouts follow the reference's own tests
+(tests/flag_attn/test_flash_attention.py:20-222).  Acceptance rule, written out: for every output
+x in {o, log-normalizer, total attention, dq, dk, dv}
+
+    max|x_hip - x_fp32| <= 2 * max|x_torch_same_precision - x_fp32| + 1e-5
+
+where both comparators come from the plain-torch oracle evaluated on the same device and inputs.
+"""
+import pytest
+import torch
+
+import flagattention_amd as flag_attn
+from oracle import flash_attention as oracle_flash, within_two_x
+
+pytestmark = pytest.mark.gpu
+
+FWD_SHAPES = [
+    (2, 4, 4, 512, 612, 128), (2, 4, 4, 1024, 1034, 64), (2, 4, 4, 2048, 2048, 32),
+    (2, 4, 4, 4096, 4096, 16), (2, 4, 4, 4001, 4001, 32), (2, 4, 4, 4001, 4096, 64),
+    (2, 4, 4, 4096, 4000, 128), (1, 2, 2, 8192, 8202, 16), (1, 2, 2, 8192, 8192, 32),
+    # grouped / multi-query heads
+    (2, 4, 2, 512, 612, 128), (2, 4, 1, 1024, 1034, 64), (2, 4, 2, 2048, 2048, 32),
+    (2, 4, 1, 4096, 4096, 16), (2, 4, 2, 4001, 4001, 32), (2, 4, 1, 4001, 4096, 64),
+    (2, 4, 2, 4096, 4000, 128), (1, 2, 1, 8192, 8202, 16), (1, 2, 1, 8192, 8192, 32),
+]
+SPLIT_SHAPES = [
+    (2, 4, 4, 1, 612, 128), (2, 4, 4, 1, 1034, 64), (2, 4, 4, 1, 2048, 32), (2, 4, 4, 1, 4096, 16),
+    (2, 4, 4, 1, 4001, 32), (2, 4, 4, 1, 4096, 64), (2, 4, 4, 2, 4000, 128), (1, 2, 2, 4, 8202, 16),
+    (1, 2, 2, 1, 8192, 32),
+    (2, 4, 2, 1, 612, 128), (2, 4, 1, 1, 1034, 64), (2, 4, 2, 1, 2048, 32), (2, 4, 1, 1, 4096, 16),
+    (2, 4, 2, 1, 4001, 32), (2, 4, 1, 1, 4096, 64), (2, 4, 2, 2, 4000, 128), (1, 2, 1, 4, 8202, 16),
+    (1, 2, 1, 1, 8192, 32),
+]
+BWD_SHAPES = [
+    (2, 4, 4, 512, 612, 128), (2, 4, 4, 1024, 1034, 64), (2, 4, 4, 2048, 2048, 32),
+    (2, 4, 4, 4096, 4096, 16), (2, 4, 4, 4001, 4001, 32), (2, 4, 4, 4001, 4096, 64),
+    (2, 4, 4, 4096, 4001, 128), (1, 2, 2, 8192, 8202, 16), (1, 2, 2, 8192, 8192, 32),
+    (2, 4, 4, 10006, 10, 128),
+    (2, 4, 2, 512, 612, 128), (2, 4, 1, 1024, 1034, 64), (2, 4, 2, 2048, 2048, 32),
+    (2, 4, 1, 4096, 4096, 16), (2, 4, 2, 4001, 4001, 32), (2, 4, 1, 4001, 4096, 64),
+    (2, 4, 2, 4096, 4001, 128), (1, 2, 1, 8192, 8202, 16), (1, 2, 1, 8192, 8192, 32),
+    (2, 4, 2, 10006, 10, 128),
+]
+AUX_SHAPES = [
+    (2, 4, 512, 612, 128), (2, 4, 1024, 1034, 64), (2, 4, 2048, 2048, 32), (2, 4, 4096, 4096, 16),
+    (2, 4, 4001, 4001, 32), (2, 4, 4001, 4096, 64), (2, 4, 4096, 4001, 128), (1, 2, 8192, 8202, 16),
+    (1, 2, 8192, 8192, 32),
+]
+
+
+def make(shape, dtype, order, std, seed, grad=False):
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    B, H, T, D = shape
+    if order == "BHTD":
+        t = torch.empty((B, H, T, D), dtype=dtype, device="cuda").normal_(0.0, std, generator=g)
+    else:
+        t = torch.empty((B, T, H, D), dtype=dtype, device="cuda").normal_(0.0, std, generator=g).transpose(1, 2)
+    return t.requires_grad_() if grad else t
+
+
+def check(name, hyp, same, ref):
+    ok, e_hyp, e_same = within_two_x(hyp, same, ref)
+    assert ok, f"{name}: hip err {e_hyp:.3e} vs same-precision torch err {e_same:.3e}"
+
+
+@pytest.mark.parametrize("scale", [1.0, 2.0, 3.0, 4.0])
+@pytest.mark.parametrize("B,Hq,Hk,M,N,D", FWD_SHAPES)
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("order", ["BHTD", "BTHD"])
+def test_attention_fwd(B, Hq, Hk, M, N, D, causal, order, dtype, scale):
+    q = make((B, Hq, M, D), dtype, order, scale, 1)
+    k = make((B, Hk, N, D), dtype, order, scale, 2)
+    v = make((B, Hk, N, D), dtype, order, scale, 3)
+    ref = oracle_flash(q, k, v, causal, upcast=True)
+    same = oracle_flash(q, k, v, causal, upcast=False)
+    hyp = flag_attn.flash_attention(q, k, v, causal)
+    assert hyp.shape == q.shape and hyp.dtype == dtype
+    check("o", hyp, same, ref)
+
+
+@pytest.mark.parametrize("scale", [10.0])
+@pytest.mark.parametrize("B,Hq,Hk,M,N,D", SPLIT_SHAPES)
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("order", ["BHTD", "BTHD"])
+def test_attention_splitkv(B, Hq, Hk, M, N, D, causal, order, dtype, scale):
+    q = make((B, Hq, M, D), dtype, order, scale, 1)
+    k = make((B, Hk, N, D), dtype, order, scale, 2)
+    v = make((B, Hk, N, D), dtype, order, scale, 3)
+    ref = oracle_flash(q, k, v, causal, upcast=True)
+    same = oracle_flash(q, k, v, causal, upcast=False)
+    hyp = flag_attn.flash_attention(q, k, v, causal)
+    check("o", hyp, same, ref)
+
+
+@pytest.mark.parametrize("scale", [1.0, 2.0, 3.0, 4.0])
+@pytest.mark.parametrize("B,Hq,Hk,M,N,D", BWD_SHAPES)
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("order", ["BHTD", "BTHD"])
+def test_attention_bwd(B, Hq, Hk, M, N, D, causal, order, dtype, scale):
+    q = make((B, Hq, M, D), dtype, order, scale, 1, grad=True)
+    k = make((B, Hk, N, D), dtype, order, scale, 2, grad=True)
+    v = make((B, Hk, N, D), dtype, order, scale, 3, grad=True)
+    do = make((B, Hq, M, D), dtype, order, 1.0, 4)
+    o_ref = oracle_flash(q, k, v, causal, upcast=True)
+    o_same = oracle_flash(q, k, v, causal, upcast=False)
+    o_hyp = flag_attn.flash_attention(q, k, v, causal)
+    g_ref = torch.autograd.grad(o_ref, (q, k, v), do)
+    g_same = torch.autograd.grad(o_same, (q, k, v), do)
+    g_hyp = torch.autograd.grad(o_hyp, (q, k, v), do)
+    check("o", o_hyp, o_same, o_ref)
+    for name, h, s, r in zip(("dq", "dk", "dv"), g_hyp, g_same, g_ref):
+        assert h.shape == r.shape
+        check(name, h, s, r)
+
+
+@pytest.mark.parametrize("scale", [1.0, 2.0, 3.0, 4.0])
+@pytest.mark.parametrize("B,H,M,N,D", AUX_SHAPES)
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("order", ["BHTD", "BTHD"])
+def test_attention_with_aux_outs(B, H, M, N, D, causal, order, dtype, scale):
+    """The reference runs this test non-causal only; the causal half is added here."""
+    q = make((B, H, M, D), dtype, order, scale, 1)
+    k = make((B, H, N, D), dtype, order, scale, 2)
+    v = make((B, H, N, D), dtype, order, scale, 3)
+    ref = oracle_flash(q, k, v, causal, upcast=True, return_log_normalizer=True, return_total_attention=True)
+    same = oracle_flash(q, k, v, causal, upcast=False, return_log_normalizer=True, return_total_attention=True)
+    o, lse, tot, seed, offset = flag_attn.flash_attention(
+        q, k, v, causal, return_log_normalizer=True, return_total_attention=True)
+    assert seed is None and offset is None
+    check("o", o, same[0], ref[0])
+    check("log_normalizer", lse, same[1], ref[1])
+    check("total_attention", tot, same[2], ref[2])
+
+
+def test_return_convention_and_asserts():
+    q = make((1, 2, 64, 32), torch.float16, "BHTD", 1.0, 1)
+    k = make((1, 2, 64, 32), torch.float16, "BHTD", 1.0, 2)
+    v = make((1, 2, 64, 32), torch.float16, "BHTD", 1.0, 3)
+    assert isinstance(flag_attn.flash_attention(q, k, v), torch.Tensor)
+    outs = flag_attn.flash_attention(q, k, v, return_log_normalizer=True)
+    assert len(outs) == 5 and outs[2] is None and outs[1].shape == (1, 2, 64)
+    with pytest.raises(AssertionError):
+        flag_attn.flash_attention(q[..., :24], k[..., :24], v[..., :24])  # head dim not in {16,32,64,128}
+    with pytest.raises(AssertionError):
+        flag_attn.flash_attention(q, k[:, :1].expand(1, 3, 64, 32), v[:, :1].expand(1, 3, 64, 32))
+    with pytest.raises(NotImplementedError):
+        flag_attn.flash_attention(q, k, v, dropout_p=0.5)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_flash_attention_split_kv_entry(causal):
+    q = make((2, 8, 1, 128), torch.float16, "BHTD", 1.0, 1)
+    k = make((2, 2, 3000, 128), torch.float16, "BHTD", 1.0, 2)
+    v = make((2, 2, 3000, 128), torch.float16, "BHTD", 1.0, 3)
+    ref = oracle_flash(q, k, v, causal, upcast=True)
+    same = oracle_flash(q, k, v, causal, upcast=False)
+    hyp = flag_attn.flash_attention_split_kv(q, k, v, causal)
+    check("o", hyp, same, ref)
