@@ -1,0 +1,219 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2]
+
+A step is one forward + backward pass of ``flash_attention`` (public API, autograd) over one batch
+of synthetic bf16 inputs that already sit in HBM.  Default workload: causal, B=1, H=32, T=8192,
+D=128 -- the configuration the target of the metric is quoted on.  ``value`` counts matmul-only
+FLOPs with the reference's convention (benchmark/flash_benchmark.py:95-103 of the reference):
+forward 4*B*H*M*N*D, backward 2.5x that, halved under the causal mask.
+
+The JSON line also carries
+  * ``roofline``: the dK/dV backward kernel (the longest launch of a step) against the dense bf16
+    MFMA peak, its launches timed with HIP events on the stream they run on;
+  * ``cpu_baseline``: the plain-torch fp32 oracle timed on the host cores on a bounded sample
+    (a few heads of the same workload);
+  * ``kernels``: every launch of a step with its own counted FLOPs and time;
+  * ``paged_decode``: the paged-attention decode configuration (64 sequences, 32 query / 8 kv heads,
+    head 128, block 16, context lengths uniform in [512, 8192]) as achieved HBM GB/s.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16/fp16 MFMA peak
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E peak
+
+# HBM traffic per launch of the dK/dV kernel at the default workload, from rocprofv3 --pmc runs
+# (FETCH_SIZE, WRITE_SIZE) scaled by a copy kernel of known size; see profiles/.  None = not measured.
+DKDV_TRAFFIC_BYTES = None
+
+WORKLOADS = {
+    "c3": dict(B=1, H=32, T=8192, D=128, name="flash_attention fwd+bwd causal bf16 B=1 H=32 T=8192 D=128"),
+    "c2": dict(B=4, H=16, T=2048, D=128, name="flash_attention fwd+bwd causal bf16 B=4 H=16 T=2048 D=128"),
+}
+
+
+def causal_pairs(M, N):
+    """Unmasked (query, key) pairs under the bottom-right aligned causal mask."""
+    if M == N:
+        return M * (M + 1) // 2
+    return sum(min(max(m + N - M + 1, 0), N) for m in range(M))
+
+
+def timed_launches(fn, iters, torch):
+    """Mean duration in ms of ``fn`` over ``iters`` launches, HIP events on the current stream."""
+    for _ in range(3):
+        fn()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(iters):
+        fn()
+    stop.record()
+    stop.synchronize()
+    return start.elapsed_time(stop) / iters
+
+
+def flash_step_bench(args, torch):
+    import flagattention_amd as flag_attn
+    from flagattention_amd import _abi, _lib
+
+    lib = _lib.get()
+    w = WORKLOADS[args.workload]
+    B, H, T, D = w["B"], w["H"], w["T"], w["D"]
+    dev = "cuda:0"
+    g = torch.Generator(device=dev).manual_seed(10086)
+    mk = lambda: torch.randn(B, H, T, D, device=dev, dtype=torch.bfloat16, generator=g)
+    q, k, v, do = mk().requires_grad_(), mk().requires_grad_(), mk().requires_grad_(), mk()
+    sm_scale = 1.0 / math.sqrt(D)
+
+    def step():
+        o = flag_attn.flash_attention(q, k, v, causal=True, sm_scale=sm_scale)
+        return torch.autograd.grad(o, (q, k, v), do)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    pairs = causal_pairs(T, T)
+    matmul = 2.0 * B * H * pairs * D          # one (T x T) x D product under the mask
+    fwd_flops, bwd_flops = 2 * matmul, 5 * matmul
+    value = (fwd_flops + bwd_flops) / (ms_per_step * 1e-3) / 1e12
+
+    # ---- per-kernel launch times (C entry points, same stream) ----
+    qd, kd, vd = q.detach(), k.detach(), v.detach()
+    o = torch.empty_like(qd)
+    lse = torch.empty(B, H, T, device=dev, dtype=torch.float32)
+    delta = torch.empty_like(lse)
+    dq, dk, dv = torch.empty_like(qd), torch.empty_like(kd), torch.empty_like(vd)
+    _abi.fa_fwd(lib, qd, kd, vd, o, lse, True, sm_scale)
+    launches = [
+        # name, callable, counted FLOPs of the launch
+        ("fa_fwd", lambda: _abi.fa_fwd(lib, qd, kd, vd, o, lse, True, sm_scale), 2 * matmul),
+        ("fa_bwd_delta", lambda: _abi.fa_bwd_delta(lib, o, do, delta), 0.0),
+        # S, dP, dV, dK: four of the five counted backward products are produced here
+        ("fa_bwd_dkdv", lambda: _abi.fa_bwd_dkdv(lib, qd, kd, vd, do, lse, delta, dk, dv, True, sm_scale), 4 * matmul),
+        # dQ; the S and dP it recomputes are not counted a second time
+        ("fa_bwd_dq", lambda: _abi.fa_bwd_dq(lib, qd, kd, vd, do, lse, delta, dq, True, sm_scale), 1 * matmul),
+    ]
+    kernels = {}
+    for name, fn, flops in launches:
+        ms = timed_launches(fn, 20, torch)
+        kernels[name] = {"ms": round(ms, 4), "counted_gflop": round(flops / 1e9, 2),
+                         "tflops": round(flops / (ms * 1e-3) / 1e12, 1) if flops else None}
+    dk_ms = kernels["fa_bwd_dkdv"]["ms"]
+    achieved = 4 * matmul / (dk_ms * 1e-3) / 1e12
+    roofline = {"kernel": "fa_bwd_dkdv_kernel", "bound": "mfma", "achieved": round(achieved, 1),
+                "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
+                "traffic": DKDV_TRAFFIC_BYTES if args.workload == "c3" else None}
+    step_frac = value / PEAK_BF16_TFLOPS
+    return w, ms_per_step, value, roofline, kernels, step_frac
+
+
+def cpu_baseline(args, torch):
+    """The fp32 oracle on the host cores over a bounded sample: 2 of the workload's heads."""
+    from oracle import flash_attention
+    w = WORKLOADS[args.workload]
+    T, D = w["T"], w["D"]
+    heads = 8 if T >= 8192 else 32
+    threads = torch.get_num_threads()
+    g = torch.Generator().manual_seed(10086)
+    mk = lambda: torch.randn(1, heads, T, D, generator=g).to(torch.bfloat16)
+    q, k, v, do = mk().requires_grad_(), mk().requires_grad_(), mk().requires_grad_(), mk()
+    best = float("inf")
+    for rep in range(2):
+        t0 = time.perf_counter()
+        for h in range(heads):  # head by head: one T x T fp32 score matrix alive at a time
+            qs, ks, vs = (t[:, h:h + 1].detach().requires_grad_() for t in (q, k, v))
+            o = flash_attention(qs, ks, vs, True, upcast=True)
+            torch.autograd.grad(o, (qs, ks, vs), do[:, h:h + 1])
+        best = min(best, time.perf_counter() - t0)
+    flops = 7 * 2.0 * heads * causal_pairs(T, T) * D
+    return {"value": round(flops / best / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": f"{heads} of {w['H'] * w['B']} (batch, head) slices of the same workload, fp32 oracle "
+                      f"fwd+bwd, best of 2, {best:.2f} s"}
+
+
+def paged_bench(torch):
+    import flagattention_amd as flag_attn
+    dev = "cuda:0"
+    g = torch.Generator(device=dev).manual_seed(10086)
+    seqs, Hq, Hkv, D, bs = 64, 32, 8, 128, 16
+    ctx = torch.randint(512, 8193, (seqs,), device=dev, generator=g, dtype=torch.int32)
+    blocks_per_seq = (ctx + bs - 1) // bs
+    num_blocks = int(blocks_per_seq.sum().item())
+    max_ctx = int(ctx.max().item())
+    max_blocks = (max_ctx + bs - 1) // bs
+    perm = torch.randperm(num_blocks, device=dev, generator=g)
+    bt = torch.zeros(seqs, max_blocks, dtype=torch.int64, device=dev)
+    start = 0
+    for s, n in enumerate(blocks_per_seq.tolist()):
+        bt[s, :n] = perm[start:start + n]
+        start += n
+    q = torch.randn(seqs, Hq, D, device=dev, dtype=torch.float16, generator=g)
+    kc = torch.randn(num_blocks, Hkv, bs, D, device=dev, dtype=torch.float16, generator=g)
+    vc = torch.randn(num_blocks, Hkv, bs, D, device=dev, dtype=torch.float16, generator=g)
+    scale = D ** -0.5
+    fn = lambda: flag_attn.paged_attention(q, kc, vc, ctx, bt, scale, max_ctx)
+    ms = timed_launches(fn, 50, torch)
+    total_ctx = int(ctx.sum().item())
+    kv_bytes = total_ctx * Hkv * D * 2 * 2
+    algo = kv_bytes + 2 * q.numel() * 2 + 8 * num_blocks
+    gbs = algo / (ms * 1e-3) / 1e9
+    return {"workload": "paged_attention decode fp16 seqs=64 Hq=32 Hkv=8 D=128 block=16 ctx~U[512,8192]",
+            "ms": round(ms, 4), "algorithmic_bytes": algo, "value": round(gbs, 1), "unit": "GB/s",
+            "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                         "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None}}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", choices=sorted(WORKLOADS), default="c3")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-paged", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (every (batch, head) slice "
+                 "is independent; see DESIGN.md for how it would shard). Run with --gpus 1.")
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU: the kernels have no CPU fallback")
+
+    w, ms, value, roofline, kernels, step_frac = flash_step_bench(args, torch)
+    out = {
+        "metric": "TFLOP/s flash_attn fwd/bwd bf16 D=128 causal; paged decode HBM GB/s",
+        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": w["name"], "batch": w["B"], "heads": w["H"], "seq_len": w["T"], "head_dim": w["D"]},
+        "frac_of_mfma_peak": round(step_frac, 4),
+        "roofline": roofline,
+        "kernels": kernels,
+    }
+    if not args.no_paged:
+        out["paged_decode"] = paged_bench(torch)
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(args, torch)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,78 @@
+"""Host-side rules of the operator wrappers: split-count rule, paged partitioning, layout checks."""
+import math
+
+import pytest
+import torch
+
+from flagattention_amd import _abi
+from flagattention_amd.paged import choose_partitioning, _next_pow2
+from flagattention_amd.split_kv import num_splits_heuristic, _split_size
+
+
+def brute_force_splits(B, H, M, N, bm, bn, cus, max_splits):
+    """The split rule written as a direct search (follows src/flag_attn/split_kv.py:234-262)."""
+    blocks = B * H * math.ceil(M / bm)
+    if blocks >= 0.8 * cus:
+        return 1
+    nb = math.ceil(N / bn)
+    cand = []
+    for s in range(1, min(cus, nb, max_splits) + 1):
+        per = math.ceil(nb / s)
+        if s == 1 or per * s - nb < per:
+            w = blocks * s / cus
+            cand.append((s, w / math.ceil(w)))
+    top = max(e for _, e in cand)
+    return next(s for s, e in cand if e >= 0.85 * top)
+
+
+@pytest.mark.parametrize("B,H,M,N", [(4, 32, 1, 32768), (2, 4, 1, 612), (1, 2, 4, 8202), (2, 4, 2, 4000),
+                                     (1, 32, 1024, 8192), (1, 1, 1, 100), (8, 8, 1, 100000)])
+@pytest.mark.parametrize("cus", [256, 108])
+def test_split_rule(B, H, M, N, cus):
+    assert num_splits_heuristic(B, H, M, N, 16, 128, cus, 128) == brute_force_splits(B, H, M, N, 16, 128, cus, 128)
+
+
+def test_known_split_counts():
+    # decode of 4 x 32 heads over 32768 keys on 256 compute units: 128 workgroups -> two splits
+    assert num_splits_heuristic(4, 32, 1, 32768, 16, 128, 256, 128) == 2
+    # a grid that already fills the device is never split
+    assert num_splits_heuristic(1, 32, 1024, 8192, 16, 128, 256, 128) == 1
+
+
+@pytest.mark.parametrize("N,S", [(32768, 2), (612, 3), (8202, 5), (100, 1)])
+def test_split_size_covers_keys_in_128_key_units(N, S):
+    size = _split_size(N, S)
+    assert size % 128 == 0 and size * S >= N and size * (S - 1) < N + 128 * S
+
+
+def test_paged_partitioning_rules():
+    for args in [(64, 8, 16, 8192, 256), (1, 8, 16, 4096, 256), (32, 64, 16, 512, 256), (1, 1, 256, 100000, 256),
+                 (16, 8, 16, 2048, 256)]:
+        splits, size = choose_partitioning(*args)
+        if splits == 1:
+            assert size == 0
+        else:
+            assert size % args[2] == 0 and size >= 512
+            assert splits == math.ceil(args[3] / size)
+    assert choose_partitioning(32, 64, 16, 512, 256) == (1, 0)   # short contexts: single pass
+    assert _next_pow2(1) == 1 and _next_pow2(5) == 8 and _next_pow2(256) == 256
+
+
+def test_kernel_ready_copies_only_when_needed():
+    a = torch.zeros(2, 3, 8, 16, dtype=torch.float16)
+    assert _abi.kernel_ready(a) is a
+    t = torch.zeros(2, 8, 3, 16, dtype=torch.float16).transpose(1, 2)  # BTHD view: still fine
+    assert _abi.kernel_ready(t) is t
+    inner = torch.zeros(2, 3, 16, 8, dtype=torch.float16).transpose(2, 3)  # inner stride != 1
+    assert _abi.kernel_ready(inner).stride(-1) == 1
+    odd = torch.zeros(2, 3, 8, 20, dtype=torch.float16)[..., :16]  # row stride 20: not a multiple of 8
+    assert _abi.kernel_ready(odd).stride(2) == 16
+    shifted = torch.zeros(2 * 3 * 8 * 16 + 4, dtype=torch.float16)[4:].view(2, 3, 8, 16)  # 8-byte aligned only
+    assert _abi.kernel_ready(shifted).data_ptr() % 16 == 0
+
+
+def test_dtype_codes():
+    assert _abi.dtype_code(torch.zeros(1, dtype=torch.float16)) == 0
+    assert _abi.dtype_code(torch.zeros(1, dtype=torch.bfloat16)) == 1
+    with pytest.raises(AssertionError):
+        _abi.dtype_code(torch.zeros(1, dtype=torch.float32))

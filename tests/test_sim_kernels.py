@@ -1,0 +1,193 @@
+"""Runs the unchanged kernel sources in the host lane simulator (tests/sim) and checks them against
+the oracle under the 2x rule.  This covers, without a GPU: tile index arithmetic, key/query tails,
+bottom-right causal masking, rows without keys, grouped heads, strided (BTHD) views, every head
+size, both dtypes, the piecewise regime switch, split merging and block-table gathers -- through the
+same C entry points and Python marshalling the GPU path uses.  Sizes are small: the simulator runs
+one lane at a time.
+"""
+import math
+
+import pytest
+import torch
+
+from flagattention_amd import _abi
+from flagattention_amd.split_kv import _split_size
+from oracle import (flash_attention, paged_attention, piecewise_attention, within_two_x)
+from tests.sim import simlib
+
+torch.manual_seed(10086)
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return simlib.get()
+
+
+def rnd(shape, dtype, bthd=False, std=1.0):
+    B, H, T, D = shape
+    if bthd:
+        return (torch.randn(B, T, H, D) * std).to(dtype).transpose(1, 2)
+    return (torch.randn(B, H, T, D) * std).to(dtype)
+
+
+def check(name, hyp, same, ref):
+    ok, e_hyp, e_same = within_two_x(hyp, same, ref)
+    assert ok, f"{name}: kernel err {e_hyp:.3e} vs same-precision torch err {e_same:.3e}"
+
+
+FLASH_CASES = [
+    # B, H, Hk, M, N, D, causal, dtype, bthd
+    (1, 2, 1, 100, 150, 128, True, torch.bfloat16, False),
+    (1, 2, 2, 130, 70, 64, True, torch.float16, True),      # M > N: rows without keys
+    (2, 2, 1, 70, 40, 32, False, torch.bfloat16, True),
+    (1, 1, 1, 33, 200, 16, True, torch.float16, False),
+    (1, 1, 1, 129, 129, 64, False, torch.bfloat16, False),
+]
+
+
+@pytest.mark.parametrize("B,H,Hk,M,N,D,causal,dtype,bthd", FLASH_CASES)
+def test_flash_forward_backward_total(lib, B, H, Hk, M, N, D, causal, dtype, bthd):
+    q = rnd((B, H, M, D), dtype, bthd).requires_grad_()
+    k = rnd((B, Hk, N, D), dtype, bthd).requires_grad_()
+    v = rnd((B, Hk, N, D), dtype, bthd).requires_grad_()
+    do = rnd((B, H, M, D), dtype, bthd)
+    sc = 1 / math.sqrt(D)
+    qd, kd, vd = q.detach(), k.detach(), v.detach()
+    o = torch.full_like(qd, float("nan"))
+    lse = torch.full((B, H, M), float("nan"))
+    _abi.fa_fwd(lib, qd, kd, vd, o, lse, causal, sc)
+    tot = torch.full((B, H, N), float("nan"))
+    _abi.fa_total_attn(lib, qd, kd, lse, tot, causal, sc)
+    delta = torch.full((B, H, M), float("nan"))
+    _abi.fa_bwd_delta(lib, o, do, delta)
+    dk = torch.full((B, H, N, D), float("nan"), dtype=dtype)
+    dv = torch.full((B, H, N, D), float("nan"), dtype=dtype)
+    dq = torch.full((B, H, M, D), float("nan"), dtype=dtype)
+    _abi.fa_bwd_dkdv(lib, qd, kd, vd, do, lse, delta, dk, dv, causal, sc)
+    _abi.fa_bwd_dq(lib, qd, kd, vd, do, lse, delta, dq, causal, sc)
+    g = H // Hk
+    dk, dv = dk.reshape(B, Hk, g, N, D).sum(2), dv.reshape(B, Hk, g, N, D).sum(2)
+
+    ref = flash_attention(q, k, v, causal, upcast=True, return_log_normalizer=True, return_total_attention=True)
+    same = flash_attention(q, k, v, causal, upcast=False, return_log_normalizer=True, return_total_attention=True)
+    g_ref = torch.autograd.grad(ref[0], (q, k, v), do)
+    g_same = torch.autograd.grad(same[0], (q, k, v), do)
+    check("o", o, same[0], ref[0])
+    check("lse", lse, same[1], ref[1])
+    check("total", tot, same[2], ref[2])
+    assert torch.allclose(delta, (o.float() * do.float()).sum(-1), atol=1e-4, rtol=1e-4)
+    for name, h, s, r in zip(("dq", "dk", "dv"), (dq, dk, dv), g_same, g_ref):
+        check(name, h, s, r)
+    if causal and M > N:
+        assert torch.all(o[:, :, : M - N] == 0) and torch.all(dq[:, :, : M - N] == 0)
+        assert torch.all(torch.isinf(lse[:, :, : M - N]))
+
+
+PW_CASES = [
+    # B, H, M, N, D, w, causal, dtype
+    (1, 2, 200, 200, 64, 50, True, torch.bfloat16),
+    (1, 1, 130, 260, 32, 100, False, torch.float16),
+    (1, 1, 260, 130, 16, 190, True, torch.bfloat16),
+    (1, 1, 150, 150, 128, -20, False, torch.float16),
+]
+
+
+@pytest.mark.parametrize("B,H,M,N,D,w,causal,dtype", PW_CASES)
+def test_piecewise_forward_backward(lib, B, H, M, N, D, w, causal, dtype):
+    ts = [rnd((B, H, M if i in (0, 2) else N, D), dtype).requires_grad_() for i in range(5)]
+    do = rnd((B, H, M, D), dtype)
+    sc = 1 / math.sqrt(D)
+    d = [t.detach() for t in ts]
+    o = torch.full_like(d[0], float("nan"))
+    lse = torch.full((B, H, M), float("nan"))
+    _abi.pw_fwd(lib, *d, o, lse, w, causal, sc)
+    delta = torch.empty(B, H, M)
+    _abi.fa_bwd_delta(lib, o, do, delta)
+    dk1, dk2, dv = (torch.full_like(d[1], float("nan")) for _ in range(3))
+    dq1, dq2 = (torch.full_like(d[0], float("nan")) for _ in range(2))
+    _abi.pw_bwd_dkdv(lib, *d, do, lse, delta, dk1, dk2, dv, w, causal, sc)
+    _abi.pw_bwd_dq(lib, *d, do, lse, delta, dq1, dq2, w, causal, sc)
+    ref = piecewise_attention(*ts, w, causal, upcast=True)
+    g_ref = torch.autograd.grad(ref, ts, do)
+    same = piecewise_attention(*ts, w, causal, upcast=False)
+    g_same = torch.autograd.grad(same, ts, do)
+    check("o", o, same, ref)
+    for name, h, s, r in zip(("dq1", "dk1", "dq2", "dk2", "dv"), (dq1, dk1, dq2, dk2, dv), g_same, g_ref):
+        check(name, h, s, r)
+
+
+SPLIT_CASES = [
+    (2, 4, 2, 1, 612, 128, False, 3, torch.float16),
+    (1, 4, 1, 2, 400, 64, True, 2, torch.bfloat16),
+    (1, 2, 2, 4, 300, 16, True, 4, torch.float16),
+    (1, 40, 1, 1, 200, 32, False, 2, torch.bfloat16),   # 40 rows share one kv head: two row blocks
+    (1, 2, 2, 40, 100, 64, True, 2, torch.float16),     # early rows see no key of the late split
+]
+
+
+@pytest.mark.parametrize("B,H,Hk,M,N,D,causal,S,dtype", SPLIT_CASES)
+def test_split_kv_and_merge(lib, B, H, Hk, M, N, D, causal, S, dtype):
+    q, k, v = rnd((B, H, M, D), dtype, std=3), rnd((B, Hk, N, D), dtype, std=3), rnd((B, Hk, N, D), dtype, std=3)
+    sc = 1 / math.sqrt(D)
+    po = torch.full((B, H, S, M, D), float("nan"), dtype=torch.float16)
+    pl = torch.full((B, H, S, M), float("nan"))
+    _abi.fa_splitkv_fwd(lib, q, k, v, po, pl, causal, sc, S, _split_size(N, S))
+    o = torch.full_like(q, float("nan"))
+    lse = torch.full((B, H, M), float("nan"))
+    _abi.fa_splitkv_combine(lib, po, pl, o, lse, S)
+    ref = flash_attention(q, k, v, causal, upcast=True, return_log_normalizer=True)
+    same = flash_attention(q, k, v, causal, upcast=False, return_log_normalizer=True)
+    check("o", o, same[0], ref[0])
+    check("lse", lse, same[1], ref[1])
+    assert not torch.isnan(po).any()
+
+
+PAGED_CASES = [
+    # seqs, Hq, G, D, block, max_len, splits, partition, dtype, table dtype
+    (3, 8, 1, 64, 16, 100, 1, 0, torch.float16, torch.int64),
+    (3, 8, 4, 128, 16, 300, 1, 0, torch.float16, torch.int64),
+    (2, 8, 8, 32, 16, 300, 3, 128, torch.float16, torch.int32),
+    (2, 4, 1, 64, 16, 2, 1, 0, torch.float16, torch.int64),
+    (2, 6, 2, 16, 32, 200, 2, 128, torch.bfloat16, torch.int64),
+    (1, 40, 40, 64, 16, 70, 2, 64, torch.float16, torch.int64),
+]
+
+
+@pytest.mark.parametrize("seqs,Hq,G,D,bs,max_len,splits,psize,dtype,tdtype", PAGED_CASES)
+def test_paged_attention_and_reduce(lib, seqs, Hq, G, D, bs, max_len, splits, psize, dtype, tdtype):
+    Hk = Hq // G
+    lens = torch.randint(1, max_len + 1, (seqs,), dtype=torch.int32)
+    lens[0] = max_len
+    nb = 50
+    sc = D ** -0.5
+    q = torch.empty(seqs, Hq, D).uniform_(-sc, sc).to(dtype)
+    kc = torch.empty(nb, Hk, bs, D).uniform_(-sc, sc).to(dtype)
+    vc = torch.empty(nb, Hk, bs, D).uniform_(-sc, sc).to(dtype)
+    bt = torch.randint(0, nb, (seqs, (max_len + bs - 1) // bs)).to(tdtype)
+    out = torch.full_like(q, float("nan"))
+    if splits == 1:
+        _abi.paged_attn(lib, out, q, kc, vc, lens, bt, sc, 0, 1, None, None, None)
+    else:
+        shape = (seqs, Hk, splits, G)
+        ml, es = torch.full(shape, float("nan")), torch.full(shape, float("nan"))
+        tmp = torch.full(shape + (D,), float("nan"), dtype=dtype)
+        _abi.paged_attn(lib, out, q, kc, vc, lens, bt, sc, psize, splits, tmp, ml, es)
+        _abi.paged_reduce(lib, out, tmp, ml, es, lens, Hk, psize, splits)
+    ref = paged_attention(q, kc, vc, bt, lens, sc)
+    same = paged_attention(q, kc, vc, bt, lens, sc, same_precision=True)
+    check("out", out, same, ref)
+    if dtype == torch.float16:
+        assert torch.allclose(out, ref, atol=2e-3, rtol=1e-5)
+
+
+def test_entry_points_reject_bad_arguments(lib):
+    q = rnd((1, 2, 32, 64), torch.float16)
+    k = rnd((1, 2, 32, 64), torch.float16)
+    o = torch.empty_like(q)
+    lse = torch.empty(1, 2, 32)
+    with pytest.raises(AssertionError):  # head size outside {16, 32, 64, 128}
+        _abi.fa_fwd(lib, q[..., :48].contiguous(), k[..., :48].contiguous(), k[..., :48].contiguous(),
+                    o[..., :48].contiguous(), lse, False, 1.0)
+    with pytest.raises(AssertionError):  # 3 query heads over 2 kv heads
+        _abi.fa_fwd(lib, rnd((1, 3, 32, 64), torch.float16), k, k, rnd((1, 3, 32, 64), torch.float16),
+                    torch.empty(1, 3, 32), False, 1.0)
