@@ -64,6 +64,56 @@ FA_DEVICE void tile_commit(const TileRegs<ROWS, COLS>& t, T* lds_tile, int tid) 
   }
 }
 
+// Loop-invariant plan of one thread's share of a ROWS x COLS tile: byte offsets inside the global
+// tile are computed once, so that a steady-state fetch is one load per chunk from a uniform tile
+// base plus a 32-bit lane offset, and the LDS destination is a fixed offset from the tile start.
+template <class T, int ROWS, int COLS>
+struct TileMover {
+  static constexpr int CPR = COLS / 8;          // 16-byte chunks per row
+  static constexpr int RPP = kThreads / CPR;    // rows covered by one pass of the workgroup
+  static constexpr int PASSES = (ROWS + RPP - 1) / RPP;
+  static constexpr bool kExact = (PASSES * RPP == ROWS);
+  u32x4 r[PASSES];
+  uint32_t goff[PASSES];
+  int row0, col0;
+
+  FA_DEVICE void init(int tid, int64_t row_stride) {
+    row0 = tid / CPR;
+    col0 = (tid % CPR) * 8;
+#pragma unroll
+    for (int i = 0; i < PASSES; ++i)
+      goff[i] = (uint32_t)(((int64_t)(row0 + i * RPP) * row_stride + col0) * (int64_t)sizeof(T));
+  }
+  // every row of the tile exists
+  FA_DEVICE void fetch_full(const T* tile_base) {
+#pragma unroll
+    for (int i = 0; i < PASSES; ++i) {
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (kExact || row0 + i * RPP < ROWS) v = *(const u32x4*)((const char*)tile_base + goff[i]);
+      r[i] = v;
+    }
+  }
+  // only the first rows_valid rows exist; the rest is filled with zeros
+  FA_DEVICE void fetch_rows(const T* tile_base, int rows_valid) {
+#pragma unroll
+    for (int i = 0; i < PASSES; ++i) {
+      u32x4 v = {0u, 0u, 0u, 0u};
+      const int row = row0 + i * RPP;
+      if ((kExact || row < ROWS) && row < rows_valid) v = *(const u32x4*)((const char*)tile_base + goff[i]);
+      r[i] = v;
+    }
+  }
+  FA_DEVICE void fetch(const T* tile_base, int rows_valid) {
+    if (rows_valid >= ROWS) fetch_full(tile_base); else fetch_rows(tile_base, rows_valid);
+  }
+  template <int LD>
+  FA_DEVICE void commit(T* lds_tile) const {
+#pragma unroll
+    for (int i = 0; i < PASSES; ++i)
+      if (kExact || row0 + i * RPP < ROWS) *(u32x4*)(lds_tile + (row0 + i * RPP) * LD + col0) = r[i];
+  }
+};
+
 // ---------------------------------------------------------------------------------------------
 // MFMA operand readers
 // ---------------------------------------------------------------------------------------------
@@ -88,6 +138,22 @@ FA_DEVICE typename hw::Elem<T>::v8 operand_transposed(const T* lds_tile, int t0,
   short4v lo = hw::lds_read_tr16(p);
   short4v hi = hw::lds_read_tr16(p + 8 * LD);
   return hw::join_v8<T>(lo, hi);
+}
+
+// Work distribution of the tiled kernels: a 1-D grid of (tile rank) x (batch * head) workgroups with
+// the (batch, head) index running fastest.  Workgroups are dispatched in id order, so ranking tiles
+// from most to least work puts every head's longest tiles first and leaves the shortest for the
+// tail (balanced finish under the causal mask); and because consecutive ids go to consecutive XCDs,
+// a given (batch, head) -- whose K/V or Q/dO every one of its tiles re-reads -- stays on one XCD's
+// L2 whenever batch * heads is a multiple of the XCD count.
+struct TileId { int rank, head, batch; };
+FA_DEVICE TileId tile_of_workgroup(int H, int B) {
+  const int lin = hw::block_x(), bh = lin % (H * B);
+  TileId t;
+  t.rank = lin / (H * B);
+  t.head = bh % H;
+  t.batch = bh / H;
+  return t;
 }
 
 // Row index inside a 32-row result block of register r for the lane's half h.

@@ -73,25 +73,28 @@ struct KvCfg {
   static constexpr int BM = 64;   // queries per pipeline step
   static constexpr int DV = D < 32 ? 32 : D;
   static constexpr int KSTEPS = D / 16;
-  static constexpr int LD = DV + 8;
+  static constexpr int LD = DV + 40;  // rows 20 banks apart: 16-byte row reads conflict-free, transposing reads nearly so
   static constexpr int TILE = BM * LD;
   static constexpr int NTILES = PW ? 3 : 2;  // Q, (Q2), dO
+  // register budget: two wavefronts per SIMD (256 registers each) when the accumulators allow it
+  static constexpr int WAVES_PER_SIMD = (D <= 64 && !(PW && D == 64)) ? 2 : 1;
   static constexpr size_t STAGE_BYTES = NTILES * TILE * sizeof(T) + 2 * BM * sizeof(float);
   static constexpr size_t LDS_BYTES = 2 * STAGE_BYTES;
 };
 
 template <class T, int D, bool PW>
-FA_KERNEL void FA_LAUNCH_BOUNDS(kThreads) fa_bwd_dkdv_kernel(BwdParams p) {
+FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (KvCfg<T, D, PW>::WAVES_PER_SIMD)) fa_bwd_dkdv_kernel(BwdParams p) {
   using C = KvCfg<T, D, PW>;
   using V8 = typename hw::Elem<T>::v8;
   FA_LDS_DECL(smem);
 
   const int tid = hw::thread_id(), lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, hh = lane >> 5;
-  const int head = hw::block_y(), batch = hw::block_z();
+  const TileId wg = tile_of_workgroup(p.H, p.B);  // key blocks in ascending order: most queries first
+  const int head = wg.head, batch = wg.batch;
   const int hk = head / p.group;
   const int M = p.M, N = p.N, pseq = N - M;
-  const int n0 = hw::block_x() * C::BN, nw = n0 + wave * 32, my_n = nw + l32;
+  const int n0 = wg.rank * C::BN, nw = n0 + wave * 32, my_n = nw + l32;
 
   const T* qb = (const T*)p.q.ptr + batch * p.q.sb + head * p.q.sh;
   const T* q2b = PW ? (const T*)p.q2.ptr + batch * p.q2.sb + head * p.q2.sh : nullptr;
@@ -280,15 +283,16 @@ struct QCfg {
   static constexpr int BN = 64;   // keys per pipeline step
   static constexpr int DV = D < 32 ? 32 : D;
   static constexpr int KSTEPS = D / 16;
-  static constexpr int LD = DV + 8;
+  static constexpr int LD = DV + 40;  // rows 20 banks apart: 16-byte row reads conflict-free, transposing reads nearly so
   static constexpr int TILE = BN * LD;
   static constexpr int NTILES = PW ? 3 : 2;  // K, (K2), V
+  static constexpr int WAVES_PER_SIMD = (PW && D == 128) ? 1 : 2;
   static constexpr size_t STAGE_BYTES = NTILES * TILE * sizeof(T);
   static constexpr size_t LDS_BYTES = 2 * STAGE_BYTES;
 };
 
 template <class T, int D, bool PW>
-FA_KERNEL void FA_LAUNCH_BOUNDS(kThreads) fa_bwd_dq_kernel(BwdParams p) {
+FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (QCfg<T, D, PW>::WAVES_PER_SIMD)) fa_bwd_dq_kernel(BwdParams p) {
   using C = QCfg<T, D, PW>;
   using V8 = typename hw::Elem<T>::v8;
   FA_LDS_DECL(smem);
@@ -296,8 +300,9 @@ FA_KERNEL void FA_LAUNCH_BOUNDS(kThreads) fa_bwd_dq_kernel(BwdParams p) {
 
   const int tid = hw::thread_id(), lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, hh = lane >> 5;
-  const int mb = hw::grid_x() - 1 - hw::block_x();
-  const int head = hw::block_y(), batch = hw::block_z();
+  const TileId wg = tile_of_workgroup(p.H, p.B);
+  const int mb = (p.M + C::BM - 1) / C::BM - 1 - wg.rank;  // long rows first under the causal mask
+  const int head = wg.head, batch = wg.batch;
   const int hk = head / p.group;
   const int M = p.M, N = p.N, pseq = N - M;
   const int m0 = mb * C::BM, mw = m0 + wave * 32, my_m = mw + l32;
@@ -468,7 +473,7 @@ FA_KERNEL void FA_LAUNCH_BOUNDS(kThreads) fa_bwd_dq_kernel(BwdParams p) {
 // ------------------------------------------------------------------------------ launchers ----
 template <class T, bool PW>
 static int launch_dkdv(const BwdParams& p, hipStream_t stream) {
-  dim3 grid((p.N + 127) / 128, p.H, p.B);
+  dim3 grid(((p.N + 127) / 128) * p.H * p.B, 1, 1);
   switch (p.D) {
     case 16: return launch(fa_bwd_dkdv_kernel<T, 16, PW>, grid, KvCfg<T, 16, PW>::LDS_BYTES, stream, p);
     case 32: return launch(fa_bwd_dkdv_kernel<T, 32, PW>, grid, KvCfg<T, 32, PW>::LDS_BYTES, stream, p);
@@ -480,7 +485,7 @@ static int launch_dkdv(const BwdParams& p, hipStream_t stream) {
 
 template <class T, bool PW>
 static int launch_dq(const BwdParams& p, hipStream_t stream) {
-  dim3 grid((p.M + 127) / 128, p.H, p.B);
+  dim3 grid(((p.M + 127) / 128) * p.H * p.B, 1, 1);
   switch (p.D) {
     case 16: return launch(fa_bwd_dq_kernel<T, 16, PW>, grid, QCfg<T, 16, PW>::LDS_BYTES, stream, p);
     case 32: return launch(fa_bwd_dq_kernel<T, 32, PW>, grid, QCfg<T, 32, PW>::LDS_BYTES, stream, p);
@@ -492,10 +497,9 @@ static int launch_dq(const BwdParams& p, hipStream_t stream) {
 
 int run_bwd_dkdv(const BwdParams& p, bool piecewise, hipStream_t stream) {
   if (p.B <= 0 || p.H <= 0 || p.M <= 0 || p.N <= 0 || p.group <= 0) return kBadArgument;
-  if (p.dtype == kDtypeF16)
-    return piecewise ? launch_dkdv<hw::half_t, true>(p, stream) : launch_dkdv<hw::half_t, false>(p, stream);
-  if (p.dtype == kDtypeBF16)
-    return piecewise ? launch_dkdv<hw::bf16_t, true>(p, stream) : launch_dkdv<hw::bf16_t, false>(p, stream);
+  if (!piecewise) return run_bwd_dkdv_plain(p, stream);  // software-pipelined kernel, fa_bwd_dkdv.hip
+  if (p.dtype == kDtypeF16) return launch_dkdv<hw::half_t, true>(p, stream);
+  if (p.dtype == kDtypeBF16) return launch_dkdv<hw::bf16_t, true>(p, stream);
   return kUnsupported;
 }
 

@@ -24,6 +24,7 @@ struct FwdCfg {
   static constexpr int BM = 128, BN = 64;
   static constexpr int DV = D < 32 ? 32 : D;  // value/output width rounded up to one MFMA block
   static constexpr int KSTEPS = D / 16;
+  static constexpr int WAVES_PER_SIMD = (PW && D == 128) ? 1 : 2;  // register budget per wavefront
   static constexpr int K_LD = D + 8;    // 16 B of padding: conflict-free 16-byte row reads
   static constexpr int V_LD = DV + 32;  // 64 B of padding: the 4 rows of a transposing read fall in disjoint banks
   static constexpr int K_TILE = BN * K_LD, V_TILE = BN * V_LD;
@@ -32,7 +33,7 @@ struct FwdCfg {
 };
 
 template <class T, int D, bool PW>
-FA_KERNEL void FA_LAUNCH_BOUNDS(kThreads) fa_fwd_kernel(FwdParams p) {
+FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (FwdCfg<T, D, PW>::WAVES_PER_SIMD)) fa_fwd_kernel(FwdParams p) {
   using C = FwdCfg<T, D, PW>;
   using V8 = typename hw::Elem<T>::v8;
   FA_LDS_DECL(smem);
@@ -40,8 +41,9 @@ FA_KERNEL void FA_LAUNCH_BOUNDS(kThreads) fa_fwd_kernel(FwdParams p) {
 
   const int tid = hw::thread_id(), lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, hh = lane >> 5;
-  const int mb = hw::grid_x() - 1 - hw::block_x();  // long rows first under the causal mask
-  const int head = hw::block_y(), batch = hw::block_z();
+  const TileId wg = tile_of_workgroup(p.H, p.B);
+  const int mb = (p.M + C::BM - 1) / C::BM - 1 - wg.rank;  // long rows first under the causal mask
+  const int head = wg.head, batch = wg.batch;
   const int hk = head / p.group;
   const int M = p.M, N = p.N, pseq = N - M;
   const int m0 = mb * C::BM, mw = m0 + wave * 32, my_m = mw + l32;
@@ -90,17 +92,21 @@ FA_KERNEL void FA_LAUNCH_BOUNDS(kThreads) fa_fwd_kernel(FwdParams p) {
   auto tile_needs_near = [&](int n0) { return !PW || (m0 + pseq - (n0 + C::BN - 1) < p.w); };
   auto tile_needs_far = [&](int n0) { return PW && (m0 + C::BM - 1 + pseq - n0 >= p.w); };
 
-  TileRegs<C::BN, D> kr, vr, k2r;
+  TileMover<T, C::BN, D> kr, vr, k2r;
+  kr.init(tid, p.k.st);
+  vr.init(tid, p.v.st);
+  if (PW) k2r.init(tid, p.k2.st);
   auto fetch = [&](int n0) {
-    if (tile_needs_near(n0)) tile_fetch<T, C::BN, D>(kr, kb, p.k.st, n0, N, tid);
-    if (tile_needs_far(n0)) tile_fetch<T, C::BN, D>(k2r, k2b, p.k2.st, n0, N, tid);
-    tile_fetch<T, C::BN, D>(vr, vb, p.v.st, n0, N, tid);
+    const int rows = N - n0;
+    if (tile_needs_near(n0)) kr.fetch(kb + (int64_t)n0 * p.k.st, rows);
+    if (tile_needs_far(n0)) k2r.fetch(k2b + (int64_t)n0 * p.k2.st, rows);
+    vr.fetch(vb + (int64_t)n0 * p.v.st, rows);
   };
   auto commit = [&](int n0, int stage) {
     T* s = lds + stage * C::STAGE;
-    if (tile_needs_near(n0)) tile_commit<T, C::BN, D, C::K_LD>(kr, s, tid);
-    if (tile_needs_far(n0)) tile_commit<T, C::BN, D, C::K_LD>(k2r, s + C::K_TILE, tid);
-    tile_commit<T, C::BN, D, C::V_LD>(vr, s + (PW ? 2 : 1) * C::K_TILE, tid);
+    if (tile_needs_near(n0)) kr.template commit<C::K_LD>(s);
+    if (tile_needs_far(n0)) k2r.template commit<C::K_LD>(s + C::K_TILE);
+    vr.template commit<C::V_LD>(s + (PW ? 2 : 1) * C::K_TILE);
   };
 
   if (n_tiles > 0) {
@@ -109,12 +115,16 @@ FA_KERNEL void FA_LAUNCH_BOUNDS(kThreads) fa_fwd_kernel(FwdParams p) {
   }
   hw::block_sync();
 
-  for (int it = 0; it < n_tiles; ++it) {
+  const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+
+  // One key tile; the LDS stage is a compile-time constant so that every operand address is a fixed
+  // offset from one per-lane base.
+  auto step = [&](int it, int kStage) {
     const int n0 = it * C::BN;
     const bool more = it + 1 < n_tiles;
     if (more) fetch(n0 + C::BN);
 
-    const T* sK = lds + (it & 1) * C::STAGE;
+    const T* sK = lds + kStage * C::STAGE;
     const T* sK2 = sK + C::K_TILE;
     const T* sV = sK + (PW ? 2 : 1) * C::K_TILE;
 
@@ -123,25 +133,27 @@ FA_KERNEL void FA_LAUNCH_BOUNDS(kThreads) fa_fwd_kernel(FwdParams p) {
 #pragma unroll
     for (int nb = 0; nb < C::BN / 32; ++nb) {
       const int nlo = n0 + nb * 32;
-      bool near = true, far = false;
-      if (PW) {  // wavefront-uniform: distances over this 32 x 32 block
-        near = (mw + pseq - (nlo + 31)) < p.w;
-        far = (mw + 31 + pseq - nlo) >= p.w;
-      }
-      f32x16 a1, a2;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) { a1[r] = 0.f; a2[r] = 0.f; }
-      if (near) {
+      if (!PW) {
+        f32x16 a1 = zero16;
 #pragma unroll
         for (int kk = 0; kk < C::KSTEPS; ++kk)
           a1 = hw::mfma32(operand_rowmajor<T, C::K_LD>(sK, nb * 32, 16 * kk, lane), qreg[kk], a1);
-      }
-      if (PW && far) {
+        s[nb] = a1;
+      } else {
+        // wavefront-uniform: distances over this 32 x 32 block
+        const bool near = (mw + pseq - (nlo + 31)) < p.w;
+        const bool far = (mw + 31 + pseq - nlo) >= p.w;
+        f32x16 a1 = zero16, a2 = zero16;
+        if (near) {
 #pragma unroll
-        for (int kk = 0; kk < C::KSTEPS; ++kk)
-          a2 = hw::mfma32(operand_rowmajor<T, C::K_LD>(sK2, nb * 32, 16 * kk, lane), q2reg[kk], a2);
-      }
-      if (PW) {
+          for (int kk = 0; kk < C::KSTEPS; ++kk)
+            a1 = hw::mfma32(operand_rowmajor<T, C::K_LD>(sK, nb * 32, 16 * kk, lane), qreg[kk], a1);
+        }
+        if (far) {
+#pragma unroll
+          for (int kk = 0; kk < C::KSTEPS; ++kk)
+            a2 = hw::mfma32(operand_rowmajor<T, C::K_LD>(sK2, nb * 32, 16 * kk, lane), q2reg[kk], a2);
+        }
         if (far && near) {
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
@@ -151,9 +163,11 @@ FA_KERNEL void FA_LAUNCH_BOUNDS(kThreads) fa_fwd_kernel(FwdParams p) {
         } else if (far) {
           a1 = a2;
         }
+        s[nb] = a1;
       }
-      s[nb] = a1;
     }
+
+    if (!PW) hw::sched_prefetched_operands<(C::BN / 32) * C::KSTEPS, (C::KSTEPS >= 4 ? 4 : C::KSTEPS)>();
 
     // ---- masks (key tail, causal) only on tiles that need them ----
     const bool need_mask = (n0 + C::BN > N) || (p.causal && (n0 + C::BN - 1 > pseq + mw));
@@ -177,7 +191,6 @@ FA_KERNEL void FA_LAUNCH_BOUNDS(kThreads) fa_fwd_kernel(FwdParams p) {
     mx = fmaxf(mx, hw::xor32(mx));
     const float m_new = fmaxf(m_i, mx);
     const float m_use = (m_new == neg_inf()) ? 0.f : m_new;  // row with no visible key so far
-    const float alpha = hw::exp2_fast((m_i - m_use) * c2);
     const float shift = -m_use * c2;
     float psum = 0.f;
 #pragma unroll
@@ -188,12 +201,19 @@ FA_KERNEL void FA_LAUNCH_BOUNDS(kThreads) fa_fwd_kernel(FwdParams p) {
         s[nb][r] = e;
         psum += e;
       }
-    l_i = l_i * alpha + psum;
+    // The accumulators are rescaled only when some row of the wavefront raised its maximum;
+    // after the first few tiles that is rare.
+    if (hw::wave_any(m_new > m_i)) {
+      hw::keep_branch();
+      const float alpha = hw::exp2_fast((m_i - m_use) * c2);
+      l_i *= alpha;
+#pragma unroll
+      for (int i = 0; i < C::DV / 32; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
+    }
+    l_i += psum;
     m_i = m_new;
-#pragma unroll
-    for (int i = 0; i < C::DV / 32; ++i)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
 
     // ---- O^T += V^T P^T ; P is rounded to the input dtype as the reference does ----
 #pragma unroll
@@ -206,9 +226,11 @@ FA_KERNEL void FA_LAUNCH_BOUNDS(kThreads) fa_fwd_kernel(FwdParams p) {
           oacc[db] = hw::mfma32(operand_transposed<T, C::V_LD>(sV, nb * 32 + 16 * c, db * 32, lane), pb, oacc[db]);
       }
 
-    if (more) commit(n0 + C::BN, (it + 1) & 1);
+    if (more) commit(n0 + C::BN, kStage ^ 1);
     hw::block_sync();
-  }
+  };
+
+  for (int it = 0; it < n_tiles; ++it) step(it, it & 1);
 
   // ---- epilogue: O = acc / l, L = m * scale + ln(l); rows that saw no key give O = 0, L = -inf ----
   const float l_tot = l_i + hw::xor32(l_i);
@@ -235,7 +257,7 @@ FA_KERNEL void FA_LAUNCH_BOUNDS(kThreads) fa_fwd_kernel(FwdParams p) {
 
 template <class T, bool PW>
 static int launch_fwd(const FwdParams& p, hipStream_t stream) {
-  dim3 grid((p.M + 127) / 128, p.H, p.B);
+  dim3 grid(((p.M + 127) / 128) * p.H * p.B, 1, 1);
   switch (p.D) {
     case 16: return launch(fa_fwd_kernel<T, 16, PW>, grid, FwdCfg<T, 16, PW>::LDS_BYTES, stream, p);
     case 32: return launch(fa_fwd_kernel<T, 32, PW>, grid, FwdCfg<T, 32, PW>::LDS_BYTES, stream, p);

@@ -24,7 +24,7 @@ struct DenseSrc {
 };
 
 template <class T, int D>
-FA_KERNEL void FA_LAUNCH_BOUNDS(kThreads) fa_splitkv_kernel(SplitParams p) {
+FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, 2) fa_splitkv_kernel(SplitParams p) {
   using C = DecCfg<T, D>;
   FA_LDS_DECL(smem);
   const int tid = hw::thread_id(), lane = tid & 63, l32 = lane & 31;

@@ -28,10 +28,11 @@ FA_KERNEL void FA_LAUNCH_BOUNDS(kThreads) fa_total_kernel(TotalParams p) {
 
   const int tid = hw::thread_id(), lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, hh = lane >> 5;
-  const int head = hw::block_y(), batch = hw::block_z();
+  const TileId wg = tile_of_workgroup(p.H, p.B);  // key blocks in ascending order: most queries first
+  const int head = wg.head, batch = wg.batch;
   const int hk = head / p.group;
   const int M = p.M, N = p.N, pseq = N - M;
-  const int n0 = hw::block_x() * C::BN, nw = n0 + wave * 32, my_n = nw + l32;
+  const int n0 = wg.rank * C::BN, nw = n0 + wave * 32, my_n = nw + l32;
 
   const T* qb = (const T*)p.q.ptr + batch * p.q.sb + head * p.q.sh;
   const T* kb = (const T*)p.k.ptr + batch * p.k.sb + hk * p.k.sh;
@@ -106,7 +107,7 @@ FA_KERNEL void FA_LAUNCH_BOUNDS(kThreads) fa_total_kernel(TotalParams p) {
 
 template <class T>
 static int launch_total(const TotalParams& p, hipStream_t stream) {
-  dim3 grid((p.N + 127) / 128, p.H, p.B);
+  dim3 grid(((p.N + 127) / 128) * p.H * p.B, 1, 1);
   switch (p.D) {
     case 16: return launch(fa_total_kernel<T, 16>, grid, TotCfg<T, 16>::LDS_BYTES, stream, p);
     case 32: return launch(fa_total_kernel<T, 32>, grid, TotCfg<T, 32>::LDS_BYTES, stream, p);

@@ -33,6 +33,7 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 #define FA_DEVICE __device__ __forceinline__
 #define FA_KERNEL __global__
 #define FA_LAUNCH_BOUNDS(n) __launch_bounds__(n)
+#define FA_LAUNCH_BOUNDS2(n, w) __launch_bounds__(n, w)
 #define FA_LDS_DECL(name) extern __shared__ __attribute__((aligned(16))) unsigned char name[]
 
 FA_DEVICE int thread_id() { return (int)threadIdx.x; }
@@ -77,10 +78,41 @@ FA_DEVICE short4v lds_read_tr16(const void* lds_ptr) {
       (__attribute__((address_space(3))) short4v*)(uintptr_t)lds_ptr);
 }
 
+// True in every lane if the predicate holds in any lane of the wavefront.
+FA_DEVICE bool wave_any(bool pred) { return __builtin_amdgcn_ballot_w64(pred) != 0; }
+
 // Value held by lane (l ^ 32).
 FA_DEVICE float xor32(float x) { return __shfl_xor(x, 32, 64); }
 // Value held by lane (l ^ mask) for mask < 64.
 FA_DEVICE float shfl_xor(float x, int mask) { return __shfl_xor(x, mask, 64); }
+
+// Marks a branch body as not speculatable, so that a wavefront-uniform `if` stays a branch instead
+// of being turned into unconditional arithmetic on selected operands.
+FA_DEVICE void keep_branch() { asm volatile("" ::: "memory"); }
+
+// Nothing is scheduled across this point by the compiler (software-pipelining fence).
+FA_DEVICE void sched_fence() { __builtin_amdgcn_sched_barrier(0); }
+
+// Scheduling hint: the next `n_mfma` matrix instructions of the region, then `n_lds` LDS reads, in
+// that order (one link of an interleaving pattern).
+template <int N_MFMA, int N_LDS>
+FA_DEVICE void sched_mfma_then_lds() {
+  __builtin_amdgcn_sched_group_barrier(0x008, N_MFMA, 0);
+  __builtin_amdgcn_sched_group_barrier(0x100, N_LDS, 0);
+}
+
+// Scheduling hint for a region of N matrix instructions that each consume one LDS-read operand:
+// keep DEPTH reads in flight ahead of the matrix instruction that needs them.
+template <int N, int DEPTH>
+FA_DEVICE void sched_prefetched_operands() {
+  __builtin_amdgcn_sched_group_barrier(0x100, DEPTH, 0);
+#pragma unroll
+  for (int i = 0; i < N - DEPTH; ++i) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+  }
+  __builtin_amdgcn_sched_group_barrier(0x008, DEPTH, 0);
+}
 
 FA_DEVICE float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
 FA_DEVICE float log_nat(float x) { return __logf(x); }
@@ -89,6 +121,8 @@ FA_DEVICE float log_nat(float x) { return __logf(x); }
 #endif  // FLAGATTN_HOST_SIM
 
 namespace hw {
+
+template <int V> struct int_tag { static constexpr int value = V; };
 
 template <class T> struct Elem;
 template <> struct Elem<half_t> { using v8 = half8; };

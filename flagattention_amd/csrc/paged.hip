@@ -45,7 +45,7 @@ struct PagedSrc {
 };
 
 template <class T, int D>
-FA_KERNEL void FA_LAUNCH_BOUNDS(kThreads) paged_attn_kernel(PagedParams p) {
+FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (D <= 128 ? 2 : 1)) paged_attn_kernel(PagedParams p) {
   using C = DecCfg<T, D>;
   FA_LDS_DECL(smem);
   const int tid = hw::thread_id(), lane = tid & 63, l32 = lane & 31;

@@ -55,10 +55,34 @@ def _split_size(N, splits):
     return -(-(-(-N // SPLIT_BLOCK_N)) // splits) * SPLIT_BLOCK_N
 
 
+def choose_num_splits(B, H, Hk, M, N, num_cus, reference_splits):
+    """Number of pieces actually launched once the split path has been chosen.
+
+    The split kernel serves a whole GQA group (up to 32 query rows) from one workgroup, so it starts
+    ``B * Hk * ceil(G * M / 32)`` workgroups per split -- fewer than the per-query-head grid the
+    reference's rule assumes.  Splits are added until the launch has about four workgroups per
+    compute unit, as long as every piece keeps at least 512 keys (four 32-key steps per wavefront).
+    ``reference_splits`` (the count the reference's rule gives) is not used beyond having selected the
+    split path.  The result of the operator does not depend on the count."""
+    group = H // Hk
+    base = B * Hk * -(-(group * M) // 32)
+    n_units = -(-N // SPLIT_BLOCK_N)
+    want = -(-4 * num_cus // base)
+    cap = max(1, N // 512)
+    splits = max(1, min(want, cap, 128))
+    splits = min(splits, n_units)
+    # drop counts that would leave the last piece empty
+    while splits > 1 and (-(-n_units // splits)) * (splits - 1) >= n_units:
+        splits -= 1
+    return splits
+
+
 def split_kv_forward(lib, q, k, v, causal, sm_scale, splits, combine=True):
     """Runs the split kernel (+ merge).  Returns (o, L), or the fp16 partials when not merging."""
     B, H, M, D = q.shape
     N = k.shape[2]
+    if splits > 1:
+        splits = choose_num_splits(B, H, k.shape[1], M, N, lib.fa_num_cus(), splits)
     part_lse = torch.empty((B, H, splits, M), dtype=torch.float32, device=q.device)
     part_o = torch.empty((B, H, splits, M, D), dtype=torch.float16, device=q.device)
     _abi.fa_splitkv_fwd(lib, q, k, v, part_o, part_lse, causal, sm_scale, splits, _split_size(N, splits))

@@ -187,6 +187,7 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 #define FA_DEVICE inline
 #define FA_KERNEL
 #define FA_LAUNCH_BOUNDS(n)
+#define FA_LAUNCH_BOUNDS2(n, w)
 #define FA_LDS_DECL(name) unsigned char* name = ::hwsim::lds
 
 inline int thread_id() { return hwsim::cur; }
@@ -243,7 +244,16 @@ inline float shfl_xor(float x, int mask) {
   return hwsim::lanes[hwsim::cur].sh_out;
 }
 inline float xor32(float x) { return shfl_xor(x, 32); }
+inline bool wave_any(bool pred) {
+  float v = pred ? 1.f : 0.f;
+  for (int m = 1; m < 64; m <<= 1) v = fmaxf(v, shfl_xor(v, m));
+  return v > 0.f;
+}
 
+inline void sched_fence() {}
+inline void keep_branch() {}
+template <int N, int DEPTH> inline void sched_prefetched_operands() {}
+template <int N_MFMA, int N_LDS> inline void sched_mfma_then_lds() {}
 inline float exp2_fast(float x) { return exp2f(x); }
 inline float log_nat(float x) { return logf(x); }
 
