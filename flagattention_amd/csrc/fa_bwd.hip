@@ -140,12 +140,16 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (KvCfg<T, D, PW>::WAVES_PER_SIMD)) fa
   auto tile_needs_near = [&](int m0) { return !PW || (m0 + pseq - (n0 + C::BN - 1) < p.w); };
   auto tile_needs_far = [&](int m0) { return PW && (m0 + C::BM - 1 + pseq - n0 >= p.w); };
 
-  TileRegs<C::BM, D> qr, q2r, gr;
+  TileMover<T, C::BM, D> qr, q2r, gr;
+  qr.init(tid, p.q.st);
+  gr.init(tid, p.dout.st);
+  if (PW) q2r.init(tid, p.q2.st);
   float l_reg = 0.f, d_reg = 0.f;
   auto fetch = [&](int m0) {
-    if (tile_needs_near(m0)) tile_fetch<T, C::BM, D>(qr, qb, p.q.st, m0, M, tid);
-    if (tile_needs_far(m0)) tile_fetch<T, C::BM, D>(q2r, q2b, p.q2.st, m0, M, tid);
-    tile_fetch<T, C::BM, D>(gr, gb, p.dout.st, m0, M, tid);
+    const int rows = M - m0;
+    if (tile_needs_near(m0)) qr.fetch(qb + (int64_t)m0 * p.q.st, rows);
+    if (tile_needs_far(m0)) q2r.fetch(q2b + (int64_t)m0 * p.q2.st, rows);
+    gr.fetch(gb + (int64_t)m0 * p.dout.st, rows);
     if (tid < C::BM) {
       int m = m0 + tid;
       // rows past M get L = +inf, hence P = 0
@@ -156,9 +160,9 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (KvCfg<T, D, PW>::WAVES_PER_SIMD)) fa
   auto commit = [&](int m0, int stage) {
     unsigned char* base = smem + stage * C::STAGE_BYTES;
     T* s = (T*)base;
-    if (tile_needs_near(m0)) tile_commit<T, C::BM, D, C::LD>(qr, s, tid);
-    if (tile_needs_far(m0)) tile_commit<T, C::BM, D, C::LD>(q2r, s + C::TILE, tid);
-    tile_commit<T, C::BM, D, C::LD>(gr, s + (C::NTILES - 1) * C::TILE, tid);
+    if (tile_needs_near(m0)) qr.template commit<C::LD>(s);
+    if (tile_needs_far(m0)) q2r.template commit<C::LD>(s + C::TILE);
+    gr.template commit<C::LD>(s + (C::NTILES - 1) * C::TILE);
     float* f = (float*)(base + C::NTILES * C::TILE * sizeof(T));
     if (tid < C::BM) { f[tid] = l_reg; f[C::BM + tid] = d_reg; }
   };
@@ -208,26 +212,41 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (KvCfg<T, D, PW>::WAVES_PER_SIMD)) fa
         dp = hw::mfma32(operand_rowmajor<T, C::LD>(sG, sb * 32, 16 * kk, lane), vreg[kk], dp);
 
       const bool need_mask = p.causal && (mr0 + pseq < nw + 31);
-      f32x16 pr, ds, ds2;
+      // L * log2e and delta of this lane's 16 query rows: rows 8g + 4h + 0..3 are contiguous
+      hw::f32x4 lrow[4], drow[4];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int ml = sb * 32 + block_row(r, hh);
-        const int m = m0 + ml;
-        float sv = s[r];
-        bool is_far = false;
-        if (PW) {
-          is_far = (m + pseq - my_n) >= p.w;
-          sv = is_far ? s2[r] : s[r];
+      for (int g = 0; g < 4; ++g) {
+        lrow[g] = *(const hw::f32x4*)(sL + sb * 32 + 8 * g + 4 * hh);
+        drow[g] = *(const hw::f32x4*)(sDl + sb * 32 + 8 * g + 4 * hh);
+      }
+      f32x16 pr, ds, ds2;
+      if (PW || need_mask) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int m = mr0 + block_row(r, hh);
+          float sv = s[r];
+          bool is_far = false;
+          if (PW) {
+            is_far = (m + pseq - my_n) >= p.w;
+            sv = is_far ? s2[r] : s[r];
+          }
+          float pv = hw::exp2_fast(fmaf(sv, c2, -lrow[r >> 2][r & 3]));
+          if (need_mask) pv = (m + pseq >= my_n) ? pv : 0.f;
+          float dsv = pv * (dp[r] - drow[r >> 2][r & 3]);
+          pr[r] = pv;
+          if (PW) {
+            ds[r] = is_far ? 0.f : dsv;
+            ds2[r] = is_far ? dsv : 0.f;
+          } else {
+            ds[r] = dsv;
+          }
         }
-        float pv = hw::exp2_fast(fmaf(sv, c2, -sL[ml]));
-        if (need_mask) pv = (m + pseq >= my_n) ? pv : 0.f;
-        float dsv = pv * (dp[r] - sDl[ml]);
-        pr[r] = pv;
-        if (PW) {
-          ds[r] = is_far ? 0.f : dsv;
-          ds2[r] = is_far ? dsv : 0.f;
-        } else {
-          ds[r] = dsv;
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float pv = hw::exp2_fast(fmaf(s[r], c2, -lrow[r >> 2][r & 3]));
+          pr[r] = pv;
+          ds[r] = pv * (dp[r] - drow[r >> 2][r & 3]);
         }
       }
 #pragma unroll
@@ -350,17 +369,21 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (QCfg<T, D, PW>::WAVES_PER_SIMD)) fa_
   auto tile_needs_near = [&](int n0) { return !PW || (m0 + pseq - (n0 + C::BN - 1) < p.w); };
   auto tile_needs_far = [&](int n0) { return PW && (m0 + C::BM - 1 + pseq - n0 >= p.w); };
 
-  TileRegs<C::BN, D> kr, k2r, vr;
+  TileMover<T, C::BN, D> kr, k2r, vr;
+  kr.init(tid, p.k.st);
+  vr.init(tid, p.v.st);
+  if (PW) k2r.init(tid, p.k2.st);
   auto fetch = [&](int n0) {
-    if (tile_needs_near(n0)) tile_fetch<T, C::BN, D>(kr, kb, p.k.st, n0, N, tid);
-    if (tile_needs_far(n0)) tile_fetch<T, C::BN, D>(k2r, k2b, p.k2.st, n0, N, tid);
-    tile_fetch<T, C::BN, D>(vr, vb, p.v.st, n0, N, tid);
+    const int rows = N - n0;
+    if (tile_needs_near(n0)) kr.fetch(kb + (int64_t)n0 * p.k.st, rows);
+    if (tile_needs_far(n0)) k2r.fetch(k2b + (int64_t)n0 * p.k2.st, rows);
+    vr.fetch(vb + (int64_t)n0 * p.v.st, rows);
   };
   auto commit = [&](int n0, int stage) {
     T* s = (T*)(smem + stage * C::STAGE_BYTES);
-    if (tile_needs_near(n0)) tile_commit<T, C::BN, D, C::LD>(kr, s, tid);
-    if (tile_needs_far(n0)) tile_commit<T, C::BN, D, C::LD>(k2r, s + C::TILE, tid);
-    tile_commit<T, C::BN, D, C::LD>(vr, s + (C::NTILES - 1) * C::TILE, tid);
+    if (tile_needs_near(n0)) kr.template commit<C::LD>(s);
+    if (tile_needs_far(n0)) k2r.template commit<C::LD>(s + C::TILE);
+    vr.template commit<C::LD>(s + (C::NTILES - 1) * C::TILE);
   };
 
   if (n_tiles > 0) { fetch(0); commit(0, 0); }
@@ -405,24 +428,29 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (QCfg<T, D, PW>::WAVES_PER_SIMD)) fa_
 
       const bool need_mask = (nlo + 32 > N) || (p.causal && (nlo + 31 > pseq + mw));
       f32x16 ds, ds2;
+      if (PW || need_mask) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int n = nlo + block_row(r, hh);
-        float sv = s[r];
-        bool is_far = false;
-        if (PW) {
-          is_far = (my_m + pseq - n) >= p.w;
-          sv = is_far ? s2[r] : s[r];
+        for (int r = 0; r < 16; ++r) {
+          const int n = nlo + block_row(r, hh);
+          float sv = s[r];
+          bool is_far = false;
+          if (PW) {
+            is_far = (my_m + pseq - n) >= p.w;
+            sv = is_far ? s2[r] : s[r];
+          }
+          float pv = hw::exp2_fast(fmaf(sv, c2, -l_row));
+          if (need_mask) pv = ((n < N) && (!p.causal || (my_m + pseq >= n))) ? pv : 0.f;
+          float dsv = pv * (dp[r] - d_row);
+          if (PW) {
+            ds[r] = is_far ? 0.f : dsv;
+            ds2[r] = is_far ? dsv : 0.f;
+          } else {
+            ds[r] = dsv;
+          }
         }
-        float pv = hw::exp2_fast(fmaf(sv, c2, -l_row));
-        if (need_mask) pv = ((n < N) && (!p.causal || (my_m + pseq >= n))) ? pv : 0.f;
-        float dsv = pv * (dp[r] - d_row);
-        if (PW) {
-          ds[r] = is_far ? 0.f : dsv;
-          ds2[r] = is_far ? dsv : 0.f;
-        } else {
-          ds[r] = dsv;
-        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) ds[r] = hw::exp2_fast(fmaf(s[r], c2, -l_row)) * (dp[r] - d_row);
       }
 #pragma unroll
       for (int c = 0; c < 2; ++c) {
@@ -497,9 +525,10 @@ static int launch_dq(const BwdParams& p, hipStream_t stream) {
 
 int run_bwd_dkdv(const BwdParams& p, bool piecewise, hipStream_t stream) {
   if (p.B <= 0 || p.H <= 0 || p.M <= 0 || p.N <= 0 || p.group <= 0) return kBadArgument;
-  if (!piecewise) return run_bwd_dkdv_plain(p, stream);  // software-pipelined kernel, fa_bwd_dkdv.hip
-  if (p.dtype == kDtypeF16) return launch_dkdv<hw::half_t, true>(p, stream);
-  if (p.dtype == kDtypeBF16) return launch_dkdv<hw::bf16_t, true>(p, stream);
+  if (p.dtype == kDtypeF16)
+    return piecewise ? launch_dkdv<hw::half_t, true>(p, stream) : launch_dkdv<hw::half_t, false>(p, stream);
+  if (p.dtype == kDtypeBF16)
+    return piecewise ? launch_dkdv<hw::bf16_t, true>(p, stream) : launch_dkdv<hw::bf16_t, false>(p, stream);
   return kUnsupported;
 }
 

@@ -59,7 +59,6 @@ namespace fa {
 int run_fwd(const FwdParams& p, bool piecewise, hipStream_t stream);
 int run_bwd_delta(const BwdParams& p, hipStream_t stream);
 int run_bwd_dkdv(const BwdParams& p, bool piecewise, hipStream_t stream);
-int run_bwd_dkdv_plain(const BwdParams& p, hipStream_t stream);  // fa_bwd_dkdv.hip
 int run_bwd_dq(const BwdParams& p, bool piecewise, hipStream_t stream);
 int run_total(const TotalParams& p, hipStream_t stream);
 }  // namespace fa
