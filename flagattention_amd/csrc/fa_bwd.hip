@@ -210,6 +210,7 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (KvCfg<T, D, PW>::WAVES_PER_SIMD)) fa
 #pragma unroll
       for (int kk = 0; kk < C::KSTEPS; ++kk)
         dp = hw::mfma32(operand_rowmajor<T, C::LD>(sG, sb * 32, 16 * kk, lane), vreg[kk], dp);
+      if (!PW) hw::sched_prefetched_operands<2 * C::KSTEPS, (C::KSTEPS >= 8 ? 8 : 2)>();
 
       const bool need_mask = p.causal && (mr0 + pseq < nw + 31);
       // L * log2e and delta of this lane's 16 query rows: rows 8g + 4h + 0..3 are contiguous
@@ -268,6 +269,8 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (KvCfg<T, D, PW>::WAVES_PER_SIMD)) fa
             dk2[db] = hw::mfma32(da2, operand_transposed<T, C::LD>(sQ2, sb * 32 + 16 * c, db * 32, lane), dk2[db]);
         }
       }
+      // each of these products takes an operand made of two transposing reads
+      if (!PW) hw::sched_prefetched_operands<4 * (C::DV / 32), (C::DV >= 128 ? 5 : 1), 2>();
     }
 
     if (more) commit(m0 + C::BM, (it + 1) & 1);
@@ -425,6 +428,7 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (QCfg<T, D, PW>::WAVES_PER_SIMD)) fa_
 #pragma unroll
       for (int kk = 0; kk < C::KSTEPS; ++kk)
         dp = hw::mfma32(operand_rowmajor<T, C::LD>(sV, nb * 32, 16 * kk, lane), greg[kk], dp);
+      if (!PW) hw::sched_prefetched_operands<2 * C::KSTEPS, (C::KSTEPS >= 4 ? 4 : 2)>();
 
       const bool need_mask = (nlo + 32 > N) || (p.causal && (nlo + 31 > pseq + mw));
       f32x16 ds, ds2;

@@ -93,23 +93,15 @@ FA_DEVICE void keep_branch() { asm volatile("" ::: "memory"); }
 // Nothing is scheduled across this point by the compiler (software-pipelining fence).
 FA_DEVICE void sched_fence() { __builtin_amdgcn_sched_barrier(0); }
 
-// Scheduling hint: the next `n_mfma` matrix instructions of the region, then `n_lds` LDS reads, in
-// that order (one link of an interleaving pattern).
-template <int N_MFMA, int N_LDS>
-FA_DEVICE void sched_mfma_then_lds() {
-  __builtin_amdgcn_sched_group_barrier(0x008, N_MFMA, 0);
-  __builtin_amdgcn_sched_group_barrier(0x100, N_LDS, 0);
-}
-
-// Scheduling hint for a region of N matrix instructions that each consume one LDS-read operand:
-// keep DEPTH reads in flight ahead of the matrix instruction that needs them.
-template <int N, int DEPTH>
+// Scheduling hint for a region of N matrix instructions that each consume an operand fetched by RPM
+// LDS reads: keep the operands of DEPTH matrix instructions in flight ahead of their consumer.
+template <int N, int DEPTH, int RPM = 1>
 FA_DEVICE void sched_prefetched_operands() {
-  __builtin_amdgcn_sched_group_barrier(0x100, DEPTH, 0);
+  __builtin_amdgcn_sched_group_barrier(0x100, DEPTH * RPM, 0);
 #pragma unroll
   for (int i = 0; i < N - DEPTH; ++i) {
     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    __builtin_amdgcn_sched_group_barrier(0x100, RPM, 0);
   }
   __builtin_amdgcn_sched_group_barrier(0x008, DEPTH, 0);
 }

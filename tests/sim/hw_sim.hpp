@@ -252,8 +252,7 @@ inline bool wave_any(bool pred) {
 
 inline void sched_fence() {}
 inline void keep_branch() {}
-template <int N, int DEPTH> inline void sched_prefetched_operands() {}
-template <int N_MFMA, int N_LDS> inline void sched_mfma_then_lds() {}
+template <int N, int DEPTH, int RPM = 1> inline void sched_prefetched_operands() {}
 inline float exp2_fast(float x) { return exp2f(x); }
 inline float log_nat(float x) { return logf(x); }
 
