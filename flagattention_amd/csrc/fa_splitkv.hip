@@ -2,7 +2,7 @@
 //
 // Replaces `_fwd_split_kv_kernel` (src/flag_attn/split_kv.py:14-160) and `_fwd_combine_kv_splits`
 // (split_kv.py:162-227).  The split kernel is the decode core of decode.hpp over a dense K/V
-// stream: a workgroup takes one (batch, kv head, split) and up to 32 of the G * M query rows that
+// stream: a workgroup takes one (batch, kv head, split) and up to 16 of the G * M query rows that
 // share that kv head, so the keys and values of a split are read once for the whole GQA group.
 // Partial outputs are fp16 whatever the input dtype, as in the reference (flash.py:96); a split
 // that holds no visible key for a row stores 0 and a log-normalizer of -inf, and the merge weights
@@ -27,7 +27,7 @@ template <class T, int D>
 FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, 2) fa_splitkv_kernel(SplitParams p) {
   using C = DecCfg<T, D>;
   FA_LDS_DECL(smem);
-  const int tid = hw::thread_id(), lane = tid & 63, l32 = lane & 31;
+  const int tid = hw::thread_id(), lane = tid & 63, li = lane & 15;
   const int rb = hw::block_x(), split = hw::block_y();
   const int batch = hw::block_z() / (p.H / p.group), hk = hw::block_z() % (p.H / p.group);
   const int M = p.M, N = p.N, pseq = N - M;
@@ -40,7 +40,7 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, 2) fa_splitkv_kernel(SplitParams p) {
   src.v_st = p.v.st;
 
   // this lane's query row: rho = g * M + m
-  const int rho = rb * 32 + l32;
+  const int rho = rb * 16 + li;
   const T* q_row = nullptr;
   int lane_limit = 0;
   if (rho < rows) {
@@ -51,15 +51,15 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, 2) fa_splitkv_kernel(SplitParams p) {
   const int n_begin = split * p.split_size;
   const int n_end = imin(N, n_begin + p.split_size);
 
-  DecodeOut<C::DV> res;
+  DecodeOut<D> res;
   decode_block<T, D>(src, q_row, n_begin, n_end, lane_limit, p.sm_scale * kLog2e, smem, res);
 
 #pragma unroll
-  for (int e = 0; e < DecodeOut<C::DV>::kPerThread; ++e) {
+  for (int e = 0; e < DecodeOut<D>::kPerThread; ++e) {
     const int idx = tid + e * kThreads;
-    const int row = idx / C::DV, d = idx % C::DV;
-    const int r = rb * 32 + row;
-    if (r < rows && d < D) {
+    const int row = idx / D, d = idx % D;
+    const int r = rb * 16 + row;
+    if (r < rows) {
       const int g = r / M, m = r % M;
       const int64_t slot = (((int64_t)batch * p.H + hk * p.group + g) * p.num_splits + split) * M + m;
       const bool empty = !(res.row_sum[e] > 0.f);
@@ -113,7 +113,7 @@ FA_KERNEL void FA_LAUNCH_BOUNDS(kThreads) fa_combine_kernel(CombineParams p) {
 template <class T>
 static int launch_split(const SplitParams& p, hipStream_t stream) {
   const int rows = p.group * p.M;
-  dim3 grid((rows + 31) / 32, p.num_splits, p.B * (p.H / p.group));
+  dim3 grid((rows + 15) / 16, p.num_splits, p.B * (p.H / p.group));
   switch (p.D) {
     case 16: return launch(fa_splitkv_kernel<T, 16>, grid, DecCfg<T, 16>::LDS_BYTES, stream, p);
     case 32: return launch(fa_splitkv_kernel<T, 32>, grid, DecCfg<T, 32>::LDS_BYTES, stream, p);

@@ -29,11 +29,8 @@ struct PagedSrc {
 #pragma unroll
     for (int i = 0; i < C::CH; ++i) {
       const int row = (lane + 64 * i) / C::CPR;
-      const int n = n0 + row;
-      int b = 0;
-      if (row < C::TK && n < n_end)
-        b = bt64 ? (int)((const int64_t*)table)[block_of(n)] : ((const int32_t*)table)[block_of(n)];
-      ids.blk[i] = b;
+      const int n = imin(n0 + row, n_end - 1);  // branch-free: rows past the end resolve the last valid token
+      ids.blk[i] = bt64 ? (int)((const int64_t*)table)[block_of(n)] : ((const int32_t*)table)[block_of(n)];
     }
   }
   FA_DEVICE const T* k_row(const Ids& ids, int i, int n) const {
@@ -48,10 +45,10 @@ template <class T, int D>
 FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (D <= 128 ? 2 : 1)) paged_attn_kernel(PagedParams p) {
   using C = DecCfg<T, D>;
   FA_LDS_DECL(smem);
-  const int tid = hw::thread_id(), lane = tid & 63, l32 = lane & 31;
+  const int tid = hw::thread_id(), lane = tid & 63, li = lane & 15;
   const int seq = hw::block_x(), hk = hw::block_y();
   const int G = p.Hq / p.Hkv;
-  const int row_blocks = (G + 31) / 32;
+  const int row_blocks = (G + 15) / 16;
   const int part = hw::block_z() / row_blocks, rb = hw::block_z() % row_blocks;
   const int ctx = p.context_lens[seq];
 
@@ -73,19 +70,19 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (D <= 128 ? 2 : 1)) paged_attn_kernel
   src.bs = p.block_size;
   src.bs_shift = (p.block_size & (p.block_size - 1)) == 0 ? __builtin_ctz(p.block_size) : -1;
 
-  const int g_lane = rb * 32 + l32;
+  const int g_lane = rb * 16 + li;
   const T* q_row = nullptr;
   if (g_lane < G) q_row = (const T*)p.q + (int64_t)seq * p.q_ss + (int64_t)(hk * G + g_lane) * p.q_sh;
 
-  DecodeOut<C::DV> res;
+  DecodeOut<D> res;
   decode_block<T, D>(src, q_row, n_begin, n_end, n_end, p.scale * kLog2e, smem, res);
 
 #pragma unroll
-  for (int e = 0; e < DecodeOut<C::DV>::kPerThread; ++e) {
+  for (int e = 0; e < DecodeOut<D>::kPerThread; ++e) {
     const int idx = tid + e * kThreads;
-    const int row = idx / C::DV, d = idx % C::DV;
-    const int g = rb * 32 + row;
-    if (g < G && d < D) {
+    const int row = idx / D, d = idx % D;
+    const int g = rb * 16 + row;
+    if (g < G) {
       const float val = res.row_sum[e] > 0.f ? res.o[e] / res.row_sum[e] : 0.f;
       if (p.partition_size > 0) {
         const int64_t slot = (((int64_t)seq * p.Hkv + hk) * p.num_parts + part) * G + g;
@@ -132,7 +129,7 @@ template <class T>
 static int launch_paged(const PagedParams& p, hipStream_t stream) {
   const int G = p.Hq / p.Hkv;
   const int parts = p.partition_size > 0 ? p.num_parts : 1;
-  dim3 grid(p.num_seqs, p.Hkv, parts * ((G + 31) / 32));
+  dim3 grid(p.num_seqs, p.Hkv, parts * ((G + 15) / 16));
   switch (p.D) {
     case 16: return launch(paged_attn_kernel<T, 16>, grid, DecCfg<T, 16>::LDS_BYTES, stream, p);
     case 32: return launch(paged_attn_kernel<T, 32>, grid, DecCfg<T, 32>::LDS_BYTES, stream, p);
