@@ -32,9 +32,12 @@ if ROOT not in sys.path:
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16/fp16 MFMA peak
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E peak
 
-# HBM traffic per launch of the dK/dV kernel at the default workload, from rocprofv3 --pmc runs
-# (FETCH_SIZE, WRITE_SIZE) scaled by a copy kernel of known size; see profiles/.  None = not measured.
-DKDV_TRAFFIC_BYTES = None
+# HBM traffic per launch at the default workloads, from rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE,
+# KiB per dispatch), each scaled by what the same counter reads for a plain 1 GiB device copy
+# (FETCH_SIZE reads 0.5 GiB for 1 GiB fetched -> x2.0; WRITE_SIZE reads 1.0 GiB -> x1.0);
+# profiles/hbm_traffic_dkdv_and_paged_pmc.txt.
+DKDV_TRAFFIC_BYTES = int((2.0 * 3.631e5 + 1.0 * 1.311e5) * 1024)    # 744 MB read + 134 MB written
+PAGED_TRAFFIC_BYTES = int((2.0 * 5.000e5 + 1.0 * 811.9) * 1024)     # 1.024 GB read + 0.8 MB written
 
 WORKLOADS = {
     "c3": dict(B=1, H=32, T=8192, D=128, name="flash_attention fwd+bwd causal bf16 B=1 H=32 T=8192 D=128"),
@@ -149,7 +152,7 @@ def cpu_baseline(args, torch):
                       f"fwd+bwd, best of 2, {best:.2f} s"}
 
 
-def paged_bench(torch):
+def paged_bench(torch, iters=50):
     import flagattention_amd as flag_attn
     dev = "cuda:0"
     g = torch.Generator(device=dev).manual_seed(10086)
@@ -170,7 +173,7 @@ def paged_bench(torch):
     vc = torch.randn(num_blocks, Hkv, bs, D, device=dev, dtype=torch.float16, generator=g)
     scale = D ** -0.5
     fn = lambda: flag_attn.paged_attention(q, kc, vc, ctx, bt, scale, max_ctx)
-    ms = timed_launches(fn, 50, torch)
+    ms = timed_launches(fn, iters, torch)
     total_ctx = int(ctx.sum().item())
     kv_bytes = total_ctx * Hkv * D * 2 * 2
     algo = kv_bytes + 2 * q.numel() * 2 + 8 * num_blocks
@@ -178,7 +181,43 @@ def paged_bench(torch):
     return {"workload": "paged_attention decode fp16 seqs=64 Hq=32 Hkv=8 D=128 block=16 ctx~U[512,8192]",
             "ms": round(ms, 4), "algorithmic_bytes": algo, "value": round(gbs, 1), "unit": "GB/s",
             "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                         "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None}}
+                         "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": PAGED_TRAFFIC_BYTES}}
+
+
+def profile_kernel(args, torch):
+    """A handful of launches of one kernel at the benchmark's shapes, nothing else on the device."""
+    from flagattention_amd import _abi, _lib
+    lib = _lib.get()
+    dev = "cuda:0"
+    if args.profile_kernel == "copy":
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"profiled": "copy", "bytes_read": 1 << 30, "bytes_written": 1 << 30}))
+        return
+    if args.profile_kernel == "paged_attn":
+        print(json.dumps({"profiled": "paged_attn", **paged_bench(torch, iters=5)}))
+        return
+    w = WORKLOADS[args.workload]
+    B, H, T, D = w["B"], w["H"], w["T"], w["D"]
+    g = torch.Generator(device=dev).manual_seed(10086)
+    mk = lambda: torch.randn(B, H, T, D, device=dev, dtype=torch.bfloat16, generator=g)
+    q, k, v, do = mk(), mk(), mk(), mk()
+    sm_scale = 1.0 / math.sqrt(D)
+    o, lse = torch.empty_like(q), torch.empty(B, H, T, device=dev, dtype=torch.float32)
+    delta = torch.empty_like(lse)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    _abi.fa_fwd(lib, q, k, v, o, lse, True, sm_scale)
+    _abi.fa_bwd_delta(lib, o, do, delta)
+    fn = {"fa_fwd": lambda: _abi.fa_fwd(lib, q, k, v, o, lse, True, sm_scale),
+          "fa_bwd_dkdv": lambda: _abi.fa_bwd_dkdv(lib, q, k, v, do, lse, delta, dk, dv, True, sm_scale),
+          "fa_bwd_dq": lambda: _abi.fa_bwd_dq(lib, q, k, v, do, lse, delta, dq, True, sm_scale)}[args.profile_kernel]
+    for _ in range(5):
+        fn()
+    torch.cuda.synchronize()
+    print(json.dumps({"profiled": args.profile_kernel, "workload": w["name"]}))
 
 
 def main():
@@ -188,6 +227,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", choices=sorted(WORKLOADS), default="c3")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--profile-kernel", choices=["fa_fwd", "fa_bwd_dkdv", "fa_bwd_dq", "paged_attn", "copy"],
+                    help="run only this launch a few times (for rocprofv3 counter passes); 'copy' is a plain "
+                         "1 GiB device copy used to calibrate FETCH_SIZE / WRITE_SIZE")
     ap.add_argument("--no-paged", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -197,6 +239,9 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU: the kernels have no CPU fallback")
 
+    if args.profile_kernel:
+        profile_kernel(args, torch)
+        return
     w, ms, value, roofline, kernels, step_frac = flash_step_bench(args, torch)
     out = {
         "metric": "TFLOP/s flash_attn fwd/bwd bf16 D=128 causal; paged decode HBM GB/s",
