@@ -156,6 +156,22 @@ def paged_attn(lib, out, query, key_cache, value_cache, context_lens, block_tabl
                          ptr(exp_sums), stream_of(query)), "paged_attn")
 
 
+def paged_attn_balanced(lib, out, query, key_cache, value_cache, context_lens, block_tables, scale,
+                        workspace, num_workgroups):
+    num_seqs, Hq, D = query.shape
+    _, Hkv, block_size, _ = key_cache.shape
+    assert block_tables.dtype in (torch.int32, torch.int64)
+    check(lib.paged_attn_balanced(dtype_code(query), ptr(out), out.stride(0), out.stride(1),
+                                  ptr(query), query.stride(0), query.stride(1),
+                                  ptr(key_cache), ptr(value_cache),
+                                  key_cache.stride(0), key_cache.stride(1), key_cache.stride(2),
+                                  ptr(context_lens), ptr(block_tables),
+                                  int(block_tables.dtype == torch.int64), block_tables.stride(0),
+                                  float(scale), num_seqs, Hq, Hkv, D, block_size, ptr(workspace),
+                                  workspace.numel() * workspace.element_size(), int(num_workgroups),
+                                  stream_of(query)), "paged_attn_balanced")
+
+
 def paged_reduce(lib, out, tmp_out, max_logits, exp_sums, context_lens, Hkv, partition_size, num_parts):
     num_seqs, Hq, D = out.shape
     check(lib.paged_reduce(dtype_code(out), ptr(out), out.stride(0), out.stride(1), ptr(tmp_out),

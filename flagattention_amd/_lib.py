@@ -36,6 +36,9 @@ SIGNATURES = {
     "paged_attn": [_i, _p, _i64, _i64, _p, _i64, _i64, _p, _p, _i64, _i64, _i64, _p, _p, _i, _i64, _f,
                    _i, _i, _i, _i, _i, _i, _i, _p, _p, _p, _p],
     "paged_reduce": [_i, _p, _i64, _i64, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p],
+    "paged_attn_balanced_workspace": [_i, _i],
+    "paged_attn_balanced": [_i, _p, _i64, _i64, _p, _i64, _i64, _p, _p, _i64, _i64, _i64, _p, _p, _i, _i64,
+                            _f, _i, _i, _i, _i, _i, _p, _i64, _i, _p],
 }
 
 

@@ -230,6 +230,40 @@ int paged_attn(int dtype, void* out, int64_t o_stride_s, int64_t o_stride_h, con
   return fa::run_paged(p, (hipStream_t)stream);
 }
 
+int paged_attn_balanced_workspace(int num_workgroups, int head_size) {
+  if (num_workgroups <= 0 || head_size <= 0) return FA_ERR_BAD_ARGUMENT;
+  const int64_t bytes = fa::paged_balanced_workspace_bytes(num_workgroups, head_size);
+  return bytes > 0x7fffffff ? FA_ERR_BAD_ARGUMENT : (int)bytes;
+}
+
+int paged_attn_balanced(int dtype, void* out, int64_t o_stride_s, int64_t o_stride_h, const void* query,
+                        int64_t q_stride_s, int64_t q_stride_h, const void* key_cache,
+                        const void* value_cache, int64_t kv_stride_blk, int64_t kv_stride_h,
+                        int64_t kv_stride_tok, const int32_t* context_lens, const void* block_tables,
+                        int bt_is_int64, int64_t bt_stride, float attn_scale, int num_seqs,
+                        int num_q_heads, int num_kv_heads, int head_size, int block_size,
+                        void* workspace, int64_t workspace_bytes, int num_workgroups, void* stream) {
+  fa::PagedParams p = {};
+  int rc = fill_paged(p, dtype, out, o_stride_s, o_stride_h, context_lens, num_seqs, num_q_heads,
+                      num_kv_heads, head_size, 0, 1, nullptr, nullptr, nullptr);
+  if (rc) return rc;
+  if (!query || !key_cache || !value_cache || !block_tables || !workspace) return FA_ERR_BAD_ARGUMENT;
+  if ((((uintptr_t)query) | ((uintptr_t)key_cache) | ((uintptr_t)value_cache) | ((uintptr_t)workspace)) & 15)
+    return FA_ERR_BAD_ARGUMENT;
+  if ((q_stride_s | q_stride_h | kv_stride_blk | kv_stride_h | kv_stride_tok) % 8) return FA_ERR_BAD_ARGUMENT;
+  if (!(head_size == 16 || head_size == 32 || head_size == 64 || head_size == 128 || head_size == 256))
+    return FA_ERR_UNSUPPORTED;
+  if (num_workgroups <= 0 || workspace_bytes < fa::paged_balanced_workspace_bytes(num_workgroups, head_size))
+    return FA_ERR_BAD_ARGUMENT;
+  p.q = query; p.q_ss = q_stride_s; p.q_sh = q_stride_h;
+  p.kc = key_cache; p.vc = value_cache;
+  p.kv_sblk = kv_stride_blk; p.kv_sh = kv_stride_h; p.kv_stok = kv_stride_tok;
+  p.block_tables = block_tables; p.bt64 = bt_is_int64; p.bt_stride = bt_stride;
+  p.scale = attn_scale; p.block_size = block_size;
+  p.ws = (float*)workspace; p.num_wgs = num_workgroups;
+  return fa::run_paged_balanced(p, (hipStream_t)stream);
+}
+
 int paged_reduce(int dtype, void* out, int64_t o_stride_s, int64_t o_stride_h, const void* tmp_out,
                  const float* max_logits, const float* exp_sums, const int32_t* context_lens,
                  int num_seqs, int num_q_heads, int num_kv_heads, int head_size, int partition_size,

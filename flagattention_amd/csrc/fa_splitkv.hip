@@ -83,20 +83,37 @@ FA_KERNEL void FA_LAUNCH_BOUNDS(kThreads) fa_combine_kernel(CombineParams p) {
   const int64_t bh = row / p.M;
   const int S = p.num_splits;
   const float* ls = p.part_lse + bh * S * p.M + m;  // stride M between splits
+  // loads of four splits are issued together: one split at a time would cost a memory latency each
+  constexpr int kBatch = 4;
   float top = neg_inf();
-  for (int s = 0; s < S; ++s) top = fmaxf(top, ls[(int64_t)s * p.M]);
+  for (int s0 = 0; s0 < S; s0 += kBatch) {
+    float t[kBatch];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) t[u] = ls[(int64_t)imin(s0 + u, S - 1) * p.M];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) top = fmaxf(top, t[u]);
+  }
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   float z = 0.f;
   if (top > neg_inf()) {
-    for (int s = 0; s < S; ++s) {
-      const float l = ls[(int64_t)s * p.M];
-      if (l == neg_inf()) continue;  // split without a visible key
-      const float wgt = hw::exp2_fast((l - top) * kLog2e);
-      z += wgt;
-      const hw::half_t* po = (const hw::half_t*)p.part_o + ((bh * S + s) * p.M + m) * D + col;
-      auto v = hw::as_v8<hw::half_t>(*(const u32x4*)po);
+    for (int s0 = 0; s0 < S; s0 += kBatch) {
+      float l[kBatch];
+      u32x4 raw[kBatch];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) acc[e] += wgt * (float)v[e];
+      for (int u = 0; u < kBatch; ++u) {
+        const int s = imin(s0 + u, S - 1);
+        l[u] = ls[(int64_t)s * p.M];
+        raw[u] = *(const u32x4*)((const hw::half_t*)p.part_o + ((bh * S + s) * p.M + m) * D + col);
+      }
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) {
+        if (s0 + u >= S || l[u] == neg_inf()) continue;  // past the end, or a split without a visible key
+        const float wgt = hw::exp2_fast((l[u] - top) * kLog2e);
+        z += wgt;
+        auto v = hw::as_v8<hw::half_t>(raw[u]);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] += wgt * (float)v[e];
+      }
     }
   }
   const float inv = z > 0.f ? 1.f / z : 0.f;

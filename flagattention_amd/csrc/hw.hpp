@@ -41,6 +41,7 @@ FA_DEVICE int block_x() { return (int)blockIdx.x; }
 FA_DEVICE int block_y() { return (int)blockIdx.y; }
 FA_DEVICE int block_z() { return (int)blockIdx.z; }
 FA_DEVICE int grid_x() { return (int)gridDim.x; }
+FA_DEVICE int grid_z() { return (int)gridDim.z; }
 FA_DEVICE void block_sync() { __syncthreads(); }
 // Orders the LDS traffic of one wavefront: writes issued by any lane before the call are visible
 // to reads issued by any lane after it (LDS serves a wavefront's requests in order; this only stops
@@ -85,6 +86,9 @@ FA_DEVICE bool wave_any(bool pred) { return __builtin_amdgcn_ballot_w64(pred) !=
 FA_DEVICE float xor32(float x) { return __shfl_xor(x, 32, 64); }
 // Value held by lane (l ^ mask) for mask < 64.
 FA_DEVICE float shfl_xor(float x, int mask) { return __shfl_xor(x, mask, 64); }
+
+// Tells the compiler that x has the same value in every lane (kept in a scalar register).
+FA_DEVICE int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
 
 // Marks a branch body as not speculatable, so that a wavefront-uniform `if` stays a branch instead
 // of being turned into unconditional arithmetic on selected operands.

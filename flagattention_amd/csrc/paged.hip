@@ -42,23 +42,7 @@ struct PagedSrc {
 };
 
 template <class T, int D>
-FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (D <= 128 ? 2 : 1)) paged_attn_kernel(PagedParams p) {
-  using C = DecCfg<T, D>;
-  FA_LDS_DECL(smem);
-  const int tid = hw::thread_id(), lane = tid & 63, li = lane & 15;
-  const int seq = hw::block_x(), hk = hw::block_y();
-  const int G = p.Hq / p.Hkv;
-  const int row_blocks = (G + 15) / 16;
-  const int part = hw::block_z() / row_blocks, rb = hw::block_z() % row_blocks;
-  const int ctx = p.context_lens[seq];
-
-  int n_begin = 0, n_end = ctx;
-  if (p.partition_size > 0) {
-    n_begin = part * p.partition_size;
-    if (n_begin >= ctx) return;  // whole workgroup: this partition lies past the context
-    n_end = imin(ctx, n_begin + p.partition_size);
-  }
-
+FA_DEVICE PagedSrc<T, D> paged_source(const PagedParams& p, int seq, int hk) {
   PagedSrc<T, D> src;
   src.kc = (const T*)p.kc + (int64_t)hk * p.kv_sh;
   src.vc = (const T*)p.vc + (int64_t)hk * p.kv_sh;
@@ -69,6 +53,32 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (D <= 128 ? 2 : 1)) paged_attn_kernel
   src.s_tok = p.kv_stok;
   src.bs = p.block_size;
   src.bs_shift = (p.block_size & (p.block_size - 1)) == 0 ? __builtin_ctz(p.block_size) : -1;
+  return src;
+}
+
+template <class T, int D>
+FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (D <= 128 ? 2 : 1)) paged_attn_kernel(PagedParams p) {
+  using C = DecCfg<T, D>;
+  FA_LDS_DECL(smem);
+  const int tid = hw::thread_id(), lane = tid & 63, li = lane & 15;
+  const int seq = hw::block_x(), hk = hw::block_y();
+  const int G = p.Hq / p.Hkv;
+  const int row_blocks = (G + 15) / 16;
+  // Partitions are issued last-first: high partitions exist only for the longest sequences, so
+  // dispatching them at the end would leave a tail in which few workgroups run; partition 0, which
+  // every sequence has, closes the launch instead.
+  const int zz = (int)hw::grid_z() - 1 - hw::block_z();
+  const int part = zz / row_blocks, rb = zz % row_blocks;
+  const int ctx = p.context_lens[seq];
+
+  int n_begin = 0, n_end = ctx;
+  if (p.partition_size > 0) {
+    n_begin = part * p.partition_size;
+    if (n_begin >= ctx) return;  // whole workgroup: this partition lies past the context
+    n_end = imin(ctx, n_begin + p.partition_size);
+  }
+
+  const PagedSrc<T, D> src = paged_source<T, D>(p, seq, hk);
 
   const int g_lane = rb * 16 + li;
   const T* q_row = nullptr;
@@ -98,6 +108,42 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (D <= 128 ? 2 : 1)) paged_attn_kernel
   }
 }
 
+// out = sum_j w_j o_j / sum_j w_j with w_j = l_j exp(m_j - max_j m_j) over n partial results of one
+// output element.  The loads of eight partials are issued together: a loop that loads, waits and
+// accumulates one partial at a time costs a full memory latency per partial.
+template <class FM, class FL, class FO>
+FA_DEVICE float merge_partials(int n, FM m_of, FL l_of, FO o_of) {
+  constexpr int kBatch = 8;
+  float top = neg_inf();
+  for (int j0 = 0; j0 < n; j0 += kBatch) {
+    float t[kBatch];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) t[u] = m_of(imin(j0 + u, n - 1));
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) top = fmaxf(top, t[u]);
+  }
+  float acc = 0.f, z = 0.f;
+  for (int j0 = 0; j0 < n; j0 += kBatch) {
+    float mv[kBatch], lv[kBatch], ov[kBatch];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const int j = imin(j0 + u, n - 1);
+      mv[u] = m_of(j);
+      lv[u] = l_of(j);
+      ov[u] = o_of(j);
+    }
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      if (j0 + u < n && lv[u] > 0.f) {
+        const float wgt = lv[u] * hw::exp2_fast((mv[u] - top) * kLog2e);
+        z += wgt;
+        acc += wgt * ov[u];
+      }
+    }
+  }
+  return z > 0.f ? acc / z : 0.f;
+}
+
 // One workgroup per (sequence, kv head): out = sum_p tmp_out_p * w_p / sum_p w_p with
 // w_p = exp_sum_p * exp(max_p - max).  Partitions past the context were never written and are skipped.
 template <class T>
@@ -110,19 +156,183 @@ FA_KERNEL void FA_LAUNCH_BOUNDS(kThreads) paged_reduce_kernel(PagedParams p) {
   const int64_t base = ((int64_t)seq * p.Hkv + hk) * p.num_parts * G;
   for (int idx = tid; idx < G * D; idx += kThreads) {
     const int g = idx / D, d = idx % D;
-    float top = neg_inf();
-    for (int s = 0; s < parts; ++s) top = fmaxf(top, p.max_logits[base + (int64_t)s * G + g]);
-    float acc = 0.f, z = 0.f;
-    for (int s = 0; s < parts; ++s) {
-      const int64_t slot = base + (int64_t)s * G + g;
-      const float l = p.exp_sums[slot];
-      if (!(l > 0.f)) continue;
-      const float wgt = l * hw::exp2_fast((p.max_logits[slot] - top) * kLog2e);
-      z += wgt;
-      acc += wgt * (float)((const T*)p.tmp_out)[slot * D + d];
-    }
-    ((T*)p.out)[(int64_t)seq * p.o_ss + (int64_t)(hk * G + g) * p.o_sh + d] = (T)(z > 0.f ? acc / z : 0.f);
+    const float val = merge_partials(
+        parts, [&](int j) { return p.max_logits[base + (int64_t)j * G + g]; },
+        [&](int j) { return p.exp_sums[base + (int64_t)j * G + g]; },
+        [&](int j) { return (float)((const T*)p.tmp_out)[(base + (int64_t)j * G + g) * D + d]; });
+    ((T*)p.out)[(int64_t)seq * p.o_ss + (int64_t)(hk * G + g) * p.o_sh + d] = (T)val;
   }
+}
+
+
+// ---------------------------------------------------------------------------------------------
+// Balanced launch: the keys of all (sequence, kv head) pairs, counted in units of 128, are laid end
+// to end and cut into num_wgs equal ranges, one per workgroup, so that every workgroup streams the
+// same number of bytes whatever the spread of context lengths and the launch is exactly one
+// resident wave of workgroups.  A pair that lies inside one range is finished by that workgroup
+// and written to `out`; a pair cut by range boundaries leaves one partial result per workgroup it
+// touches (at most two per workgroup: the pair it starts in the middle of, slot 2w, and the pair it
+// leaves unfinished, slot 2w + 1), which paged_balanced_reduce_kernel merges.
+//
+// Workspace (floats): 2 * num_wgs slots of [16][D] normalised outputs, [16] max logits, [16] sums of
+// exponentials; then num_wgs records of 4 ints {sequence, kv head, row block, number of following
+// workgroups that continue the pair left unfinished} (the last is 0 when there is no such pair).
+// ---------------------------------------------------------------------------------------------
+constexpr int kUnitKeys = 128;
+constexpr int kMinUnitsPerWg = 2;
+
+template <int D> FA_DEVICE int balanced_slot_floats() { return 16 * D + 32; }
+
+template <class T, int D>
+FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (D <= 128 ? 2 : 1)) paged_balanced_kernel(PagedParams p) {
+  using C = DecCfg<T, D>;
+  FA_LDS_DECL(smem);
+  const int tid = hw::thread_id(), lane = tid & 63, li = lane & 15;
+  const int w = hw::block_x();
+  const int G = p.Hq / p.Hkv;
+  const int row_blocks = (G + 15) / 16;
+  const int pairs_per_seq = p.Hkv * row_blocks;
+  auto units_of = [&](int seq) { const int c = p.context_lens[seq]; return c > 0 ? (c + kUnitKeys - 1) / kUnitKeys : 0; };
+
+  // ---- every workgroup scans the context lengths (num_seqs values, served from L2) ----
+  const int chunk = cdiv(p.num_seqs, kThreads);
+  const int s_lo = imin(p.num_seqs, tid * chunk), s_hi = imin(p.num_seqs, s_lo + chunk);
+  int mine = 0;
+  for (int s = s_lo; s < s_hi; ++s) {
+    const int u = units_of(s);
+    mine += u;
+    if (u == 0 && w == 0) {  // an empty sequence has no keys to stream: its output rows are zero
+      for (int i = 0; i < p.Hq * D; ++i) ((T*)p.out)[(int64_t)s * p.o_ss + (int64_t)(i / D) * p.o_sh + i % D] = (T)0.f;
+    }
+  }
+  int* scan_a = (int*)smem;
+  int* scan_b = scan_a + kThreads;
+  int* found = scan_b + kThreads;  // {first sequence of this workgroup, units before it}
+  scan_a[tid] = mine;
+  hw::block_sync();
+  for (int off = 1; off < kThreads; off <<= 1) {
+    const int v = scan_a[tid] + (tid >= off ? scan_a[tid - off] : 0);
+    scan_b[tid] = v;
+    hw::block_sync();
+    int* t = scan_a; scan_a = scan_b; scan_b = t;
+  }
+  const int64_t total = (int64_t)scan_a[kThreads - 1] * pairs_per_seq;
+  const int64_t per = (int64_t)imax(kMinUnitsPerWg, (int)((total + p.num_wgs - 1) / p.num_wgs));
+  const int64_t u_begin = (int64_t)w * per;
+  const int64_t u_end = u_begin + per < total ? u_begin + per : total;
+  int* meta = (int*)(p.ws + (int64_t)2 * p.num_wgs * balanced_slot_floats<D>()) + 4 * w;
+  if (u_begin >= total) {  // whole workgroup
+    if (tid == 0) meta[3] = 0;
+    return;
+  }
+  {
+    const int incl = scan_a[tid], excl = incl - mine;
+    if ((int64_t)excl * pairs_per_seq <= u_begin && u_begin < (int64_t)incl * pairs_per_seq) {
+      int pre = excl;
+      for (int s = s_lo; s < s_hi; ++s) {
+        const int u = units_of(s);
+        if (u_begin < (int64_t)(pre + u) * pairs_per_seq) { found[0] = s; found[1] = pre; break; }
+        pre += u;
+      }
+    }
+  }
+  hw::block_sync();
+  int seq = hw::uniform(found[0]);
+  int before = hw::uniform(found[1]);
+  int64_t u = u_begin;
+  int unfinished = 0;
+
+  while (u < u_end) {
+    const int ctx = hw::uniform(p.context_lens[seq]);
+    const int us = ctx > 0 ? (ctx + kUnitKeys - 1) / kUnitKeys : 0;
+    const int local = (int)(u - (int64_t)before * pairs_per_seq);  // unit index inside this sequence's pairs
+    if (us == 0 || local >= us * pairs_per_seq) { before += us; ++seq; continue; }
+    const int pr = local / us, lo = local % us;
+    const int hk = pr / row_blocks, rb = pr % row_blocks;
+    const int hi = (int)(u_end - u < (int64_t)(us - lo) ? lo + (u_end - u) : us);
+    const int n_begin = lo * kUnitKeys, n_end = imin(ctx, hi * kUnitKeys);
+
+    const PagedSrc<T, D> src = paged_source<T, D>(p, seq, hk);
+    const int g_lane = rb * 16 + li;
+    const T* q_row = nullptr;
+    if (g_lane < G) q_row = (const T*)p.q + (int64_t)seq * p.q_ss + (int64_t)(hk * G + g_lane) * p.q_sh;
+
+    hw::block_sync();  // the scan, or the previous pair's merge area, is read out before staging reuses it
+    DecodeOut<D> res;
+    decode_block<T, D>(src, q_row, n_begin, n_end, n_end, p.scale * kLog2e, smem, res);
+
+    const bool whole = lo == 0 && hi == us;
+    float* slot = p.ws + (int64_t)(2 * w + (lo == 0 ? 1 : 0)) * balanced_slot_floats<D>();
+#pragma unroll
+    for (int e = 0; e < DecodeOut<D>::kPerThread; ++e) {
+      const int idx = tid + e * kThreads;
+      const int row = idx / D, d = idx % D;
+      const int g = rb * 16 + row;
+      if (idx < 16 * D && g < G) {
+        const float val = res.row_sum[e] > 0.f ? res.o[e] / res.row_sum[e] : 0.f;
+        if (whole) {
+          ((T*)p.out)[(int64_t)seq * p.o_ss + (int64_t)(hk * G + g) * p.o_sh + d] = (T)val;
+        } else {
+          slot[row * D + d] = val;
+          if (d == 0) {
+            slot[16 * D + row] = res.row_max[e] * p.scale;
+            slot[16 * D + 16 + row] = res.row_sum[e];
+          }
+        }
+      }
+    }
+    if (lo == 0 && hi < us) {  // this pair continues in the following workgroups, `per` units each
+      unfinished = (int)(((int64_t)(us - hi) + per - 1) / per);
+      if (tid == 0) { meta[0] = seq; meta[1] = hk; meta[2] = rb; }
+    }
+    u += hi - lo;
+  }
+  if (tid == 0) meta[3] = unfinished;
+}
+
+// Workgroup w merges the pair that attention workgroup w started and left unfinished: slot 2w + 1
+// and slot 2(w + j) of each of the following workgroups that continued it.
+template <class T, int D>
+FA_KERNEL void FA_LAUNCH_BOUNDS(kThreads) paged_balanced_reduce_kernel(PagedParams p) {
+  const int tid = hw::thread_id();
+  const int w = hw::block_x();
+  const int SF = balanced_slot_floats<D>();
+  const int* meta = (const int*)(p.ws + (int64_t)2 * p.num_wgs * SF) + 4 * w;
+  const int follow = meta[3];
+  if (follow <= 0) return;
+  const int seq = meta[0], hk = meta[1], rb = meta[2];
+  const int G = p.Hq / p.Hkv;
+  for (int idx = tid; idx < 16 * D; idx += kThreads) {
+    const int row = idx / D, d = idx % D;
+    const int g = rb * 16 + row;
+    if (g >= G) continue;
+    auto slot_of = [&](int j) { return p.ws + (int64_t)(j == 0 ? 2 * w + 1 : 2 * (w + j)) * SF; };
+    const float val = merge_partials(
+        follow + 1, [&](int j) { return slot_of(j)[16 * D + row]; },
+        [&](int j) { return slot_of(j)[16 * D + 16 + row]; }, [&](int j) { return slot_of(j)[row * D + d]; });
+    ((T*)p.out)[(int64_t)seq * p.o_ss + (int64_t)(hk * G + g) * p.o_sh + d] = (T)val;
+  }
+}
+
+template <class T, int D>
+static int launch_balanced_d(const PagedParams& p, hipStream_t stream) {
+  dim3 grid(p.num_wgs, 1, 1);
+  const size_t lds = DecCfg<T, D>::LDS_BYTES > 4096 ? DecCfg<T, D>::LDS_BYTES : 4096;
+  int rc = launch(paged_balanced_kernel<T, D>, grid, lds, stream, p);
+  if (rc) return rc;
+  return launch(paged_balanced_reduce_kernel<T, D>, grid, 0, stream, p);
+}
+
+template <class T>
+static int launch_balanced(const PagedParams& p, hipStream_t stream) {
+  switch (p.D) {
+    case 16: return launch_balanced_d<T, 16>(p, stream);
+    case 32: return launch_balanced_d<T, 32>(p, stream);
+    case 64: return launch_balanced_d<T, 64>(p, stream);
+    case 128: return launch_balanced_d<T, 128>(p, stream);
+    case 256: return launch_balanced_d<T, 256>(p, stream);
+  }
+  return kUnsupported;
 }
 
 template <class T>
@@ -151,6 +361,17 @@ int run_paged(const PagedParams& p, hipStream_t stream) {
   if (!paged_args_ok(p)) return kBadArgument;
   if (p.dtype == kDtypeF16) return launch_paged<hw::half_t>(p, stream);
   if (p.dtype == kDtypeBF16) return launch_paged<hw::bf16_t>(p, stream);
+  return kUnsupported;
+}
+
+int64_t paged_balanced_workspace_bytes(int num_wgs, int D) {
+  return (int64_t)num_wgs * (2 * (16 * (int64_t)D + 32) * (int64_t)sizeof(float) + 4 * (int64_t)sizeof(int));
+}
+
+int run_paged_balanced(const PagedParams& p, hipStream_t stream) {
+  if (!paged_args_ok(p) || p.partition_size != 0 || p.num_wgs <= 0 || !p.ws) return kBadArgument;
+  if (p.dtype == kDtypeF16) return launch_balanced<hw::half_t>(p, stream);
+  if (p.dtype == kDtypeBF16) return launch_balanced<hw::bf16_t>(p, stream);
   return kUnsupported;
 }
 

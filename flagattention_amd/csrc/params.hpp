@@ -98,11 +98,15 @@ struct PagedParams {
   int partition_size, num_parts;
   void* tmp_out; float* max_logits; float* exp_sums;
   int dtype;
+  // balanced launch only: partial results of workgroups that share a (sequence, kv head) pair
+  float* ws; int num_wgs;
 };
 
 int run_splitkv(const SplitParams& p, hipStream_t stream);
 int run_combine(const CombineParams& p, hipStream_t stream);
 int run_paged(const PagedParams& p, hipStream_t stream);
 int run_paged_reduce(const PagedParams& p, hipStream_t stream);
+int64_t paged_balanced_workspace_bytes(int num_wgs, int D);
+int run_paged_balanced(const PagedParams& p, hipStream_t stream);
 
 }  // namespace fa

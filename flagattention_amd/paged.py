@@ -17,24 +17,20 @@ def _next_pow2(x):
     return 1 << max(0, (int(x) - 1).bit_length())
 
 
-def choose_partitioning(num_seqs, num_kv_heads, block_size, max_context_len, num_cus):
-    """Automatic partitioning for ``num_splits == 0`` on a device with ``num_cus`` compute units.
+def choose_launch(num_seqs, num_kv_heads, group, head_size, max_context_len, num_cus):
+    """Launch shape for ``num_splits == 0`` on a device with ``num_cus`` compute units.
 
-    One workgroup handles one (sequence, kv head, partition).  Partitions are cut so that the launch
-    has about four workgroups per compute unit when the batch alone cannot provide them, but never
-    shorter than 512 tokens (each wavefront then still streams four 32-key steps) and always a
-    multiple of the cache block size.  Returns (num_splits, partition_size); num_splits == 1 means a
-    single pass that writes the output directly."""
-    pairs = num_seqs * num_kv_heads
-    if max_context_len <= 1024 or pairs >= 8 * num_cus:
-        return 1, 0
-    want = max(1, -(-4 * num_cus // pairs))
-    size = max(512, _next_pow2(-(-max_context_len // want)))
-    size = -(-size // block_size) * block_size
-    splits = -(-max_context_len // size)
-    if splits <= 1:
-        return 1, 0
-    return splits, size
+    Returns ("balanced", num_workgroups) or ("single", 0).  The balanced launch divides the keys of
+    all (sequence, kv head) pairs evenly over one resident wave of workgroups (two per compute unit
+    fit up to head size 128, one at 256) and so does not depend on how the context lengths are
+    spread; its fixed cost (a scan of the context lengths per workgroup, a merge kernel) only loses
+    against one workgroup per pair when there are many more short pairs than workgroups, where the
+    hardware's own dispatch already evens things out."""
+    num_wgs = num_cus * (2 if head_size <= 128 else 1)
+    pairs = num_seqs * num_kv_heads * (-(-group // 16))
+    if pairs >= 8 * num_wgs and max_context_len <= 2048:
+        return "single", 0
+    return "balanced", num_wgs
 
 
 def attention(query, key_cache, value_cache, context_lens, block_tables, attn_scale,
@@ -62,9 +58,16 @@ def attention(query, key_cache, value_cache, context_lens, block_tables, attn_sc
 
     with torch.cuda.device(query.device):
         if num_splits == 0:
-            num_splits, partition_size = choose_partitioning(
-                num_seqs, num_kv_heads, block_size, max_context_len, lib.fa_num_cus())
-        elif num_splits > 1:
+            kind, num_wgs = choose_launch(num_seqs, num_kv_heads, group, head_size, max_context_len,
+                                          lib.fa_num_cus())
+            if kind == "balanced":
+                nbytes = lib.paged_attn_balanced_workspace(num_wgs, head_size)
+                workspace = torch.empty(nbytes // 4, dtype=torch.float32, device=query.device)
+                _abi.paged_attn_balanced(lib, out, query, key_cache, value_cache, context_lens,
+                                         block_tables, attn_scale, workspace, num_wgs)
+                return out
+            num_splits = 1
+        if num_splits > 1:
             partition_size = _next_pow2(-(-max_context_len // num_splits))
             assert partition_size >= block_size and partition_size % block_size == 0, \
                 f"partition_size={partition_size}, kv_block_size={block_size}"

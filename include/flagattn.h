@@ -133,6 +133,24 @@ int paged_reduce(int dtype, void* out, int64_t o_stride_s, int64_t o_stride_h, c
                  int num_seqs, int num_q_heads, int num_kv_heads, int head_size, int partition_size,
                  int num_parts, void* stream);
 
+
+/* paged_attn_balanced <- the automatic choice of partitions in `attention` (paged.py:44-56, the
+ * `num_splits == 0` branch) together with the two launches it leads to (:57-162).  Instead of
+ * cutting every sequence into partitions of one size, the keys of all (sequence, kv head) pairs are
+ * laid end to end and divided evenly over num_workgroups workgroups (use twice the number of compute
+ * units for head_size <= 128, once for 256); pairs cut by a boundary are merged by a second kernel
+ * launched by the same call.  `workspace` is device memory of at least
+ * paged_attn_balanced_workspace(num_workgroups, head_size) bytes, 16-byte aligned; its contents on
+ * entry do not matter and it may be reused by the next call on the same stream. */
+int paged_attn_balanced_workspace(int num_workgroups, int head_size);
+int paged_attn_balanced(int dtype, void* out, int64_t o_stride_s, int64_t o_stride_h, const void* query,
+                        int64_t q_stride_s, int64_t q_stride_h, const void* key_cache,
+                        const void* value_cache, int64_t kv_stride_blk, int64_t kv_stride_h,
+                        int64_t kv_stride_tok, const int32_t* context_lens, const void* block_tables,
+                        int bt_is_int64, int64_t bt_stride, float attn_scale, int num_seqs,
+                        int num_q_heads, int num_kv_heads, int head_size, int block_size,
+                        void* workspace, int64_t workspace_bytes, int num_workgroups, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

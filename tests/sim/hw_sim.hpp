@@ -49,7 +49,7 @@ inline ucontext_t sched_ctx;
 inline void* sched_fake = nullptr;
 inline const void* sched_bottom = nullptr;
 inline size_t sched_size = 0;
-inline int bx, by, bz, gx;
+inline int bx, by, bz, gx, gz;
 inline unsigned char* lds = nullptr;
 inline std::function<void()> body;
 
@@ -125,6 +125,7 @@ inline void run_grid(dim3 grid, int threads, size_t lds_bytes, std::function<voi
   if (threads % 64) die("workgroup size must be a multiple of the wavefront size");
   body = fn;
   gx = (int)grid.x;
+  gz = (int)grid.z;
   lanes.resize(threads);
   for (auto& ln : lanes)
     if (!ln.stack) ln.stack = (char*)malloc(kStack);
@@ -195,6 +196,8 @@ inline int block_x() { return hwsim::bx; }
 inline int block_y() { return hwsim::by; }
 inline int block_z() { return hwsim::bz; }
 inline int grid_x() { return hwsim::gx; }
+inline int uniform(int x) { return x; }
+inline int grid_z() { return hwsim::gz; }
 inline void block_sync() { hwsim::yield(hwsim::OP_BARRIER); }
 inline void wave_sync() { hwsim::yield(hwsim::OP_WAVESYNC); }
 

@@ -5,7 +5,7 @@ import pytest
 import torch
 
 from flagattention_amd import _abi
-from flagattention_amd.paged import choose_partitioning, _next_pow2
+from flagattention_amd.paged import choose_launch, _next_pow2
 from flagattention_amd.split_kv import num_splits_heuristic, _split_size
 
 
@@ -45,16 +45,14 @@ def test_split_size_covers_keys_in_128_key_units(N, S):
     assert size % 128 == 0 and size * S >= N and size * (S - 1) < N + 128 * S
 
 
-def test_paged_partitioning_rules():
-    for args in [(64, 8, 16, 8192, 256), (1, 8, 16, 4096, 256), (32, 64, 16, 512, 256), (1, 1, 256, 100000, 256),
-                 (16, 8, 16, 2048, 256)]:
-        splits, size = choose_partitioning(*args)
-        if splits == 1:
-            assert size == 0
-        else:
-            assert size % args[2] == 0 and size >= 512
-            assert splits == math.ceil(args[3] / size)
-    assert choose_partitioning(32, 64, 16, 512, 256) == (1, 0)   # short contexts: single pass
+def test_paged_launch_choice():
+    # (num_seqs, kv heads, group, head size, max context, compute units)
+    assert choose_launch(64, 8, 4, 128, 8192, 256) == ("balanced", 512)
+    assert choose_launch(1, 8, 4, 128, 32768, 256) == ("balanced", 512)
+    assert choose_launch(32, 16, 1, 256, 8192, 256) == ("balanced", 256)   # one workgroup per CU at 256
+    assert choose_launch(2048, 8, 4, 128, 1024, 256) == ("single", 0)      # many short pairs
+    assert choose_launch(2048, 8, 4, 128, 4096, 256) == ("balanced", 512)  # long contexts: keep balancing
+    assert choose_launch(100, 1, 40, 64, 1024, 256) == ("balanced", 512)   # 3 row blocks per kv head
     assert _next_pow2(1) == 1 and _next_pow2(5) == 8 and _next_pow2(256) == 256
 
 

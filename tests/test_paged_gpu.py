@@ -84,3 +84,53 @@ def test_baseline_decode_configuration_small_copy():
     """The BASELINE decode configuration (32 query heads over 8 kv heads, head 128, block 16) at a
     reduced number of sequences so that the token-gather oracle stays fast."""
     run_case(8, 32, 4, 128, 16, 8192)
+
+
+def test_many_short_pairs_take_the_single_pass_launch():
+    from flagattention_amd.paged import choose_launch
+    assert choose_launch(700, 64, 1, 64, 300, 256)[0] == "single"
+    run_case(700, 64, 1, 64, 16, 300)
+
+
+def test_balanced_launch_skewed_contexts_with_an_empty_sequence():
+    g = torch.Generator(device="cuda").manual_seed(3)
+    num_seqs, Hq, Hkv, D, bs = 9, 16, 4, 128, 16
+    context_lens = torch.tensor([5000, 1, 0, 129, 2047, 16, 0, 3001, 640], dtype=torch.int32, device="cuda")
+    scale = D ** -0.5
+    q = torch.empty(num_seqs, Hq, D, dtype=torch.float16, device="cuda").uniform_(-scale, scale, generator=g)
+    k_cache = torch.empty(NUM_BLOCKS, Hkv, bs, D, dtype=torch.float16, device="cuda").uniform_(-scale, scale, generator=g)
+    v_cache = torch.empty_like(k_cache).uniform_(-scale, scale, generator=g)
+    block_tables = torch.randint(0, NUM_BLOCKS, (num_seqs, (5000 + bs - 1) // bs), device="cuda", generator=g)
+    out = flag_attn.paged_attention(q, k_cache, v_cache, context_lens, block_tables, scale, 5000)
+    live = context_lens > 0
+    assert (out[~live] == 0).all()
+    ref = oracle_paged(q[live], k_cache, v_cache, block_tables[live], context_lens[live], scale)
+    same = oracle_paged(q[live], k_cache, v_cache, block_tables[live], context_lens[live], scale, same_precision=True)
+    assert torch.allclose(out[live], ref, atol=2e-3, rtol=1e-5)
+    ok, e_hyp, e_same = within_two_x(out[live], same, ref)
+    assert ok, f"hip err {e_hyp:.3e} vs same-precision torch err {e_same:.3e}"
+
+
+def test_full_size_decode_launch_shapes_agree():
+    """At the benchmark's size (64 sequences, contexts U[512, 8192], 32 query heads over 8 kv heads,
+    head 128) the oracle's token gather is too slow, but how the keys are cut into pieces must not
+    matter: the balanced launch, one pass and 4 or 16 partitions give the same output up to the fp16
+    rounding of the partial results, and 8 sequences of it are checked against the oracle."""
+    g = torch.Generator(device="cuda").manual_seed(10086)
+    num_seqs, Hq, Hkv, D, bs = 64, 32, 8, 128, 16
+    context_lens = torch.randint(512, 8193, (num_seqs,), dtype=torch.int32, device="cuda", generator=g)
+    blocks_per_seq = (context_lens + bs - 1) // bs
+    num_blocks = int(blocks_per_seq.sum())
+    max_context_len = int(context_lens.max())
+    scale = D ** -0.5
+    q = torch.empty(num_seqs, Hq, D, dtype=torch.float16, device="cuda").uniform_(-scale, scale, generator=g)
+    k_cache = torch.empty(num_blocks, Hkv, bs, D, dtype=torch.float16, device="cuda").uniform_(-scale, scale, generator=g)
+    v_cache = torch.empty_like(k_cache).uniform_(-scale, scale, generator=g)
+    block_tables = torch.randint(0, num_blocks, (num_seqs, (max_context_len + bs - 1) // bs), device="cuda", generator=g)
+    outs = [flag_attn.paged_attention(q, k_cache, v_cache, context_lens, block_tables, scale, max_context_len, n)
+            for n in (0, 1, 4, 16)]
+    for o in outs[1:]:
+        assert torch.allclose(outs[0].float(), o.float(), atol=1e-3, rtol=0)
+    sub = slice(0, 8)
+    ref = oracle_paged(q[sub], k_cache, v_cache, block_tables[sub], context_lens[sub], scale)
+    assert torch.allclose(outs[0][sub], ref, atol=2e-3, rtol=1e-5)

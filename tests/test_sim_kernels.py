@@ -180,6 +180,41 @@ def test_paged_attention_and_reduce(lib, seqs, Hq, G, D, bs, max_len, splits, ps
         assert torch.allclose(out, ref, atol=2e-3, rtol=1e-5)
 
 
+BALANCED_CASES = [
+    # seqs, Hq, G, D, block, lens, workgroups, dtype, table dtype
+    (4, 4, 2, 64, 16, [700, 1, 300, 129], 7, torch.float16, torch.int64),   # pairs cut at both ends
+    (3, 2, 1, 128, 16, [1000, 0, 260], 3, torch.float16, torch.int32),      # an empty sequence
+    (2, 40, 40, 32, 8, [200, 90], 4, torch.bfloat16, torch.int64),          # 3 row blocks per kv head
+    (5, 2, 2, 16, 16, [40, 50, 60, 70, 80], 64, torch.float16, torch.int64),  # more workgroups than work
+    (1, 2, 1, 64, 16, [1500], 5, torch.float16, torch.int64),               # one pair over many workgroups
+]
+
+
+@pytest.mark.parametrize("seqs,Hq,G,D,bs,lens,wgs,dtype,tdtype", BALANCED_CASES)
+def test_paged_attention_balanced(lib, seqs, Hq, G, D, bs, lens, wgs, dtype, tdtype):
+    Hk = Hq // G
+    lens = torch.tensor(lens, dtype=torch.int32)
+    max_len = int(lens.max())
+    nb = 120
+    sc = D ** -0.5
+    q = torch.empty(seqs, Hq, D).uniform_(-sc, sc).to(dtype)
+    kc = torch.empty(nb, Hk, bs, D).uniform_(-sc, sc).to(dtype)
+    vc = torch.empty(nb, Hk, bs, D).uniform_(-sc, sc).to(dtype)
+    bt = torch.randint(0, nb, (seqs, (max_len + bs - 1) // bs)).to(tdtype)
+    out = torch.full_like(q, float("nan"))
+    nbytes = lib.paged_attn_balanced_workspace(wgs, D)
+    assert nbytes > 0
+    ws = torch.full((nbytes // 4,), float("nan"))
+    _abi.paged_attn_balanced(lib, out, q, kc, vc, lens, bt, sc, ws, wgs)
+    live = lens > 0
+    assert (out[~live] == 0).all()
+    ref = paged_attention(q[live], kc, vc, bt[live], lens[live], sc)
+    same = paged_attention(q[live], kc, vc, bt[live], lens[live], sc, same_precision=True)
+    check("out", out[live], same, ref)
+    if dtype == torch.float16:
+        assert torch.allclose(out[live], ref, atol=2e-3, rtol=1e-5)
+
+
 def test_entry_points_reject_bad_arguments(lib):
     q = rnd((1, 2, 32, 64), torch.float16)
     k = rnd((1, 2, 32, 64), torch.float16)
