@@ -36,8 +36,9 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E peak
 # KiB per dispatch), each scaled by what the same counter reads for a plain 1 GiB device copy
 # (FETCH_SIZE reads 0.5 GiB for 1 GiB fetched -> x2.0; WRITE_SIZE reads 1.0 GiB -> x1.0);
 # profiles/hbm_traffic_dkdv_and_paged_pmc.txt.
-DKDV_TRAFFIC_BYTES = int((2.0 * 3.631e5 + 1.0 * 1.311e5) * 1024)    # 744 MB read + 134 MB written
-PAGED_TRAFFIC_BYTES = int((2.0 * 5.000e5 + 1.0 * 811.9) * 1024)     # 1.024 GB read + 0.8 MB written
+DKDV_TRAFFIC_BYTES = int((2.0 * 3.631e5 + 1.0 * 1.311e5) * 1024)      # recomputing path: 744 MB read + 134 MB written
+DKDV_DS_TRAFFIC_BYTES = int((2.0 * 3.639e5 + 1.0 * 2.236e6) * 1024)   # dS kept: 745 MB read + 2.29 GB written
+PAGED_TRAFFIC_BYTES = int((2.0 * 5.014e5 + 1.0 * 4010) * 1024)        # 1.027 GB read + 4 MB written
 
 WORKLOADS = {
     "c3": dict(B=1, H=32, T=8192, D=128, name="flash_attention fwd+bwd causal bf16 B=1 H=32 T=8192 D=128"),
@@ -105,25 +106,43 @@ def flash_step_bench(args, torch):
     delta = torch.empty_like(lse)
     dq, dk, dv = torch.empty_like(qd), torch.empty_like(kd), torch.empty_like(vd)
     _abi.fa_fwd(lib, qd, kd, vd, o, lse, True, sm_scale)
+    from flagattention_amd.flash import ds_heads_per_launch
     launches = [
         # name, callable, counted FLOPs of the launch
         ("fa_fwd", lambda: _abi.fa_fwd(lib, qd, kd, vd, o, lse, True, sm_scale), 2 * matmul),
         ("fa_bwd_delta", lambda: _abi.fa_bwd_delta(lib, o, do, delta), 0.0),
-        # S, dP, dV, dK: four of the five counted backward products are produced here
-        ("fa_bwd_dkdv", lambda: _abi.fa_bwd_dkdv(lib, qd, kd, vd, do, lse, delta, dk, dv, True, sm_scale), 4 * matmul),
-        # dQ; the S and dP it recomputes are not counted a second time
-        ("fa_bwd_dq", lambda: _abi.fa_bwd_dq(lib, qd, kd, vd, do, lse, delta, dq, True, sm_scale), 1 * matmul),
     ]
+    if ds_heads_per_launch(lib, B, H, 1, T, T, D) >= B * H:   # the launches the backward above made
+        ds = torch.empty(lib.fa_bwd_ds_workspace_mib(B, H, T, T) << 20, dtype=torch.uint8, device=dev)
+        dkdv_name = "fa_bwd_dkdv_ds"
+        launches += [
+            # S, dP, dV, dK: four of the five counted backward products are produced here; dS is kept
+            (dkdv_name, lambda: _abi.fa_bwd_dkdv_ds(lib, qd, kd, vd, do, lse, delta, dk, dv, ds, True, sm_scale), 4 * matmul),
+            # dQ = dS K: the fifth product, bound by reading dS back
+            ("fa_bwd_dq_from_ds", lambda: _abi.fa_bwd_dq_from_ds(lib, kd, ds, dq, True, sm_scale), 1 * matmul),
+        ]
+    else:
+        dkdv_name = "fa_bwd_dkdv"
+        launches += [
+            (dkdv_name, lambda: _abi.fa_bwd_dkdv(lib, qd, kd, vd, do, lse, delta, dk, dv, True, sm_scale), 4 * matmul),
+            # dQ; the S and dP it recomputes are not counted a second time
+            ("fa_bwd_dq", lambda: _abi.fa_bwd_dq(lib, qd, kd, vd, do, lse, delta, dq, True, sm_scale), 1 * matmul),
+        ]
     kernels = {}
     for name, fn, flops in launches:
         ms = timed_launches(fn, 20, torch)
         kernels[name] = {"ms": round(ms, 4), "counted_gflop": round(flops / 1e9, 2),
                          "tflops": round(flops / (ms * 1e-3) / 1e12, 1) if flops else None}
-    dk_ms = kernels["fa_bwd_dkdv"]["ms"]
+    if "fa_bwd_dq_from_ds" in kernels:   # algorithmic bytes: the visible dS blocks once, k and dq once
+        ds_bytes = B * H * pairs * 2 + 2 * qd.numel() * 2
+        kernels["fa_bwd_dq_from_ds"]["hbm_gbs"] = round(ds_bytes / (kernels["fa_bwd_dq_from_ds"]["ms"] * 1e-3) / 1e9, 1)
+    dk_ms = kernels[dkdv_name]["ms"]
     achieved = 4 * matmul / (dk_ms * 1e-3) / 1e12
-    roofline = {"kernel": "fa_bwd_dkdv_kernel", "bound": "mfma", "achieved": round(achieved, 1),
+    roofline = {"kernel": dkdv_name + "_kernel" if dkdv_name == "fa_bwd_dkdv" else "fa_bwd_dkdv_kernel (dS kept)",
+                "bound": "mfma", "achieved": round(achieved, 1),
                 "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
-                "traffic": DKDV_TRAFFIC_BYTES if args.workload == "c3" else None}
+                "traffic": None if args.workload != "c3" else
+                (DKDV_DS_TRAFFIC_BYTES if dkdv_name == "fa_bwd_dkdv_ds" else DKDV_TRAFFIC_BYTES)}
     step_frac = value / PEAK_BF16_TFLOPS
     return w, ms_per_step, value, roofline, kernels, step_frac
 
@@ -211,8 +230,12 @@ def profile_kernel(args, torch):
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     _abi.fa_fwd(lib, q, k, v, o, lse, True, sm_scale)
     _abi.fa_bwd_delta(lib, o, do, delta)
+    ds = torch.empty(lib.fa_bwd_ds_workspace_mib(B, H, T, T) << 20, dtype=torch.uint8, device=dev)
+    _abi.fa_bwd_dkdv_ds(lib, q, k, v, do, lse, delta, dk, dv, ds, True, sm_scale)
     fn = {"fa_fwd": lambda: _abi.fa_fwd(lib, q, k, v, o, lse, True, sm_scale),
           "fa_bwd_dkdv": lambda: _abi.fa_bwd_dkdv(lib, q, k, v, do, lse, delta, dk, dv, True, sm_scale),
+          "fa_bwd_dkdv_ds": lambda: _abi.fa_bwd_dkdv_ds(lib, q, k, v, do, lse, delta, dk, dv, ds, True, sm_scale),
+          "fa_bwd_dq_from_ds": lambda: _abi.fa_bwd_dq_from_ds(lib, k, ds, dq, True, sm_scale),
           "fa_bwd_dq": lambda: _abi.fa_bwd_dq(lib, q, k, v, do, lse, delta, dq, True, sm_scale)}[args.profile_kernel]
     for _ in range(5):
         fn()
@@ -227,7 +250,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", choices=sorted(WORKLOADS), default="c3")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--profile-kernel", choices=["fa_fwd", "fa_bwd_dkdv", "fa_bwd_dq", "paged_attn", "copy"],
+    ap.add_argument("--profile-kernel", choices=["fa_fwd", "fa_bwd_dkdv", "fa_bwd_dkdv_ds", "fa_bwd_dq", "fa_bwd_dq_from_ds",
+                                                  "paged_attn", "copy"],
                     help="run only this launch a few times (for rocprofv3 counter passes); 'copy' is a plain "
                          "1 GiB device copy used to calibrate FETCH_SIZE / WRITE_SIZE")
     ap.add_argument("--no-paged", action="store_true")

@@ -104,6 +104,22 @@ def fa_bwd_dq(lib, q, k, v, do, lse, delta, dq, causal, sm_scale):
           "fa_bwd_dq")
 
 
+def fa_bwd_dkdv_ds(lib, q, k, v, do, lse, delta, dk, dv, ds, causal, sm_scale):
+    B, H, M, D = q.shape
+    Hk, N = k.shape[1], k.shape[2]
+    check(lib.fa_bwd_dkdv_ds(dtype_code(q), view4(q), view4(k), view4(v), view4(do), ptr(lse), ptr(delta),
+                             view4(dk), view4(dv), ptr(ds), ds.numel() * ds.element_size(), B, H, Hk, M,
+                             N, D, int(causal), float(sm_scale), stream_of(q)), "fa_bwd_dkdv_ds")
+
+
+def fa_bwd_dq_from_ds(lib, k, ds, dq, causal, sm_scale):
+    B, H, M, D = dq.shape
+    Hk, N = k.shape[1], k.shape[2]
+    check(lib.fa_bwd_dq_from_ds(dtype_code(dq), view4(k), ptr(ds), ds.numel() * ds.element_size(),
+                                view4(dq), B, H, Hk, M, N, D, int(causal), float(sm_scale),
+                                stream_of(dq)), "fa_bwd_dq_from_ds")
+
+
 def pw_bwd_dkdv(lib, q1, k1, q2, k2, v, do, lse, delta, dk1, dk2, dv, w, causal, sm_scale):
     B, H, M, D = q1.shape
     N = k1.shape[2]

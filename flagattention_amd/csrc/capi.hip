@@ -120,6 +120,45 @@ int fa_bwd_dq(int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v
   return fa::run_bwd_dq(p, false, (hipStream_t)stream);
 }
 
+int fa_bwd_ds_workspace_mib(int B, int H, int M, int N) {
+  if (B <= 0 || H <= 0 || M <= 0 || N <= 0) return FA_ERR_BAD_ARGUMENT;
+  const int64_t mib = (fa::bwd_ds_workspace_bytes(B, H, M, N) + (1 << 20) - 1) >> 20;
+  return mib > 0x7fffffff ? FA_ERR_BAD_ARGUMENT : (int)mib;
+}
+
+int fa_bwd_dkdv_ds(int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v,
+                   const fa_view4* dout, const float* lse, const float* delta, const fa_view4* dk,
+                   const fa_view4* dv, void* ds_workspace, int64_t ds_workspace_bytes, int B, int H,
+                   int Hk, int M, int N, int D, int causal, float sm_scale, void* stream) {
+  fa::BwdParams p = {};
+  int rc = fill_bwd(p, dtype, q, k, v, dout, lse, delta, B, H, Hk, M, N, D, causal, sm_scale);
+  if (rc) return rc;
+  if (!view_ok(dk) || !view_ok(dv)) return FA_ERR_BAD_ARGUMENT;
+  if (!ds_workspace || (((uintptr_t)ds_workspace) & 15) ||
+      ds_workspace_bytes < fa::bwd_ds_workspace_bytes(B, H, M, N))
+    return FA_ERR_BAD_ARGUMENT;
+  p.dk = to_view(dk); p.dv = to_view(dv);
+  p.ds = ds_workspace;
+  return fa::run_bwd_dkdv_ds(p, (hipStream_t)stream);
+}
+
+int fa_bwd_dq_from_ds(int dtype, const fa_view4* k, const void* ds_workspace, int64_t ds_workspace_bytes,
+                      const fa_view4* dq, int B, int H, int Hk, int M, int N, int D, int causal,
+                      float sm_scale, void* stream) {
+  if (!view_ok(k) || !view_ok(dq)) return FA_ERR_BAD_ARGUMENT;
+  if (!head_dim_ok(D)) return FA_ERR_UNSUPPORTED;
+  if (B <= 0 || H <= 0 || Hk <= 0 || H % Hk || M <= 0 || N <= 0) return FA_ERR_BAD_ARGUMENT;
+  if (!ds_workspace || (((uintptr_t)ds_workspace) & 15) ||
+      ds_workspace_bytes < fa::bwd_ds_workspace_bytes(B, H, M, N))
+    return FA_ERR_BAD_ARGUMENT;
+  fa::BwdParams p = {};
+  p.k = to_view(k); p.dq = to_view(dq);
+  p.ds = const_cast<void*>(ds_workspace);
+  p.B = B; p.H = H; p.M = M; p.N = N; p.D = D; p.group = H / Hk;
+  p.causal = causal; p.sm_scale = sm_scale; p.dtype = dtype;
+  return fa::run_bwd_dq_from_ds(p, (hipStream_t)stream);
+}
+
 int pw_bwd_dkdv(int dtype, const fa_view4* q1, const fa_view4* k1, const fa_view4* q2,
                 const fa_view4* k2, const fa_view4* v, const fa_view4* dout, const float* lse,
                 const float* delta, const fa_view4* dk1, const fa_view4* dk2, const fa_view4* dv,

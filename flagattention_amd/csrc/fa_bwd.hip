@@ -82,7 +82,11 @@ struct KvCfg {
   static constexpr size_t LDS_BYTES = 2 * STAGE_BYTES;
 };
 
-template <class T, int D, bool PW>
+// DS: also leave dS (rounded to T, as it enters dK += dS^T Q) in the workspace p.ds for
+// fa_bwd_dq_from_ds_kernel, one 2 KB chunk per 32 x 32 block in the order the MFMA result holds it:
+// chunk[c][lane] = 8 elements, queries 16c + 8g + 4(lane / 32) + e at position 4g + e, key lane % 32.
+// Chunks are indexed (batch * H + head, key block, query block); both counts padded to 4.
+template <class T, int D, bool PW, bool DS = false>
 FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (KvCfg<T, D, PW>::WAVES_PER_SIMD)) fa_bwd_dkdv_kernel(BwdParams p) {
   using C = KvCfg<T, D, PW>;
   using V8 = typename hw::Elem<T>::v8;
@@ -139,6 +143,13 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (KvCfg<T, D, PW>::WAVES_PER_SIMD)) fa
 
   auto tile_needs_near = [&](int m0) { return !PW || (m0 + pseq - (n0 + C::BN - 1) < p.w); };
   auto tile_needs_far = [&](int m0) { return PW && (m0 + C::BM - 1 + pseq - n0 >= p.w); };
+
+  // dS chunks of this wavefront's key block: one row of the (key block, query block) chunk grid
+  T* ds_row = nullptr;
+  if (DS) {
+    const int64_t nqb = 4 * (int64_t)cdiv(M, 128), nkb = 4 * (int64_t)cdiv(N, 128);
+    ds_row = (T*)p.ds + ((((int64_t)batch * p.H + head) * nkb + (n0 / 32 + wave)) * nqb) * 1024 + lane * 8;
+  }
 
   TileMover<T, C::BM, D> qr, q2r, gr;
   qr.init(tid, p.q.st);
@@ -258,6 +269,7 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (KvCfg<T, D, PW>::WAVES_PER_SIMD)) fa
           dv[db] = hw::mfma32(pa, operand_transposed<T, C::LD>(sG, sb * 32 + 16 * c, db * 32, lane), dv[db]);
         if (near) {
           V8 da = pack_half_block<T>(ds, c);
+          if (DS) hw::store_streaming(ds_row + (int64_t)(mr0 / 32) * 1024 + c * 512, __builtin_bit_cast(u32x4, da));
 #pragma unroll
           for (int db = 0; db < C::DV / 32; ++db)
             dk[db] = hw::mfma32(da, operand_transposed<T, C::LD>(sQ, sb * 32 + 16 * c, db * 32, lane), dk[db]);
@@ -502,6 +514,146 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (QCfg<T, D, PW>::WAVES_PER_SIMD)) fa_
   }
 }
 
+
+// --------------------------------------------------------------------------- dQ from dS ----
+// dQ = scale * dS K with dS read back from the workspace the dK/dV kernel left (see there for the
+// chunk format) instead of being recomputed: one product instead of three and no exponentials,
+// paid for with one write and one read of the B x H x M x N matrix in T -- a trade that HBM3E
+// bandwidth makes worthwhile.  The kernel is bound by that read.
+//
+// A wavefront owns 32 queries and walks the keys in steps of 64.  Its own dS chunks (2 per step) go
+// through a private LDS patch verbatim; the transposing read then hands lane (query, h) the keys
+// t0 + 4h + 0..3 and t0 + 8 + 4h + 0..3 of a 16-key slice, the order in which the K^T operand
+// (operand_transposed) lists them.  In the patch the two halves of a chunk vector (lanes 0..31 and
+// 32..63 of the writer) are 64 bytes further apart than in memory, which keeps the 16 lanes of a
+// transposing read in distinct banks.
+template <class T, int D>
+struct QdsCfg {
+  static constexpr int BM = 128, BN = 64;
+  static constexpr int DV = D < 32 ? 32 : D;
+  static constexpr int LD = DV + 40;
+  static constexpr int TILE = BN * LD;                 // K tile, elements
+  static constexpr int VEC = 512 + 32 + 32;            // one chunk vector in the patch: 2 x (256 + 32 pad) elements
+  static constexpr int PATCH = 2 * 2 * VEC;            // 2 chunks x 2 vectors per wavefront and stage
+  static constexpr size_t STAGE_BYTES = (TILE + 4 * PATCH) * sizeof(T);
+  static constexpr size_t LDS_BYTES = 2 * STAGE_BYTES;
+};
+
+template <class T, int D>
+FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, 2) fa_bwd_dq_from_ds_kernel(BwdParams p) {
+  using C = QdsCfg<T, D>;
+  using V8 = typename hw::Elem<T>::v8;
+  FA_LDS_DECL(smem);
+  T* lds = (T*)smem;
+
+  const int tid = hw::thread_id(), lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, hh = lane >> 5;
+  const TileId wg = tile_of_workgroup(p.H, p.B);
+  const int mb = (p.M + C::BM - 1) / C::BM - 1 - wg.rank;  // long rows first under the causal mask
+  const int head = wg.head, batch = wg.batch;
+  const int hk = head / p.group;
+  const int M = p.M, N = p.N, pseq = N - M;
+  const int m0 = mb * C::BM, mw = m0 + wave * 32, my_m = mw + l32;
+  const bool live = mw < M;  // wavefront has at least one query row
+
+  const T* kb = (const T*)p.k.ptr + batch * p.k.sb + hk * p.k.sh;
+  const int64_t nqb = 4 * (int64_t)cdiv(M, 128), nkb = 4 * (int64_t)cdiv(N, 128);
+  // chunk (key block 0, this wavefront's query block); a key block further is nqb chunks further
+  const T* ds_col = (const T*)p.ds + ((((int64_t)batch * p.H + head) * nkb) * nqb + mw / 32) * 1024 + lane * 8;
+
+  int hi = N;
+  if (p.causal) hi = imin(N, pseq + m0 + C::BM);
+  const int n_tiles = hi > 0 ? cdiv(hi, C::BN) : 0;
+
+  if (C::DV != D) {
+    for (int i = tid; i < (int)(C::LDS_BYTES / sizeof(T)); i += kThreads) lds[i] = (T)0.f;
+    hw::block_sync();
+  }
+
+  f32x16 dq[C::DV / 32];
+#pragma unroll
+  for (int i = 0; i < C::DV / 32; ++i)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) dq[i][r] = 0.f;
+
+  // a 32-key block contributes unless the mask hides all of it from this wavefront's rows
+  auto block_used = [&](int nlo) { return live && !(p.causal && (mw + 31 + pseq < nlo)); };
+
+  TileMover<T, C::BN, D> kr;
+  kr.init(tid, p.k.st);
+  u32x4 dsr[2][2];
+  auto fetch = [&](int n0) {
+    kr.fetch(kb + (int64_t)n0 * p.k.st, N - n0);
+    // unconditional: chunks the mask hides were never written, are in bounds, and are not used below
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) {
+      const T* chunk = ds_col + (int64_t)(n0 / 32 + nb) * nqb * 1024;
+      dsr[nb][0] = hw::load_streaming(chunk);
+      dsr[nb][1] = hw::load_streaming(chunk + 512);
+    }
+  };
+  // patch position of what writer lane l (= this lane) stored: half l / 32 starts 288 elements on
+  const int patch_off = l32 * 8 + hh * (256 + 32);
+  auto commit = [&](int stage) {
+    T* s = (T*)(smem + stage * C::STAGE_BYTES);
+    kr.template commit<C::LD>(s);
+    T* patch = s + C::TILE + wave * C::PATCH;
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) {
+      *(u32x4*)(patch + (2 * nb + 0) * C::VEC + patch_off) = dsr[nb][0];
+      *(u32x4*)(patch + (2 * nb + 1) * C::VEC + patch_off) = dsr[nb][1];
+    }
+  };
+  // Supplier role of this lane in a transposing read (16-lane group G = lane / 16, row r = lane % 16 =
+  // 4e + a): it points at key t0 + 4 (G / 2) + e of the queries 16 (G % 2) + 4a + 0..3, which the
+  // writer kept in vector G % 2, half a % 2, elements 4 (a / 2) + 0..3.
+  const int G = lane >> 4, r = lane & 15, e4 = r >> 2, a = r & 3;
+  const int tr_off = (G & 1) * C::VEC + (a & 1) * (256 + 32) + (4 * (G >> 1) + e4) * 8 + 4 * (a >> 1);
+
+  if (n_tiles > 0) { fetch(0); commit(0); }
+  hw::block_sync();
+
+  for (int it = 0; it < n_tiles; ++it) {
+    const int n0 = it * C::BN;
+    const bool more = it + 1 < n_tiles;
+    if (more) fetch(n0 + C::BN);
+
+    const T* sK = (const T*)(smem + (it & 1) * C::STAGE_BYTES);
+    const T* patch = sK + C::TILE + wave * C::PATCH;
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) {
+      if (!block_used(n0 + 32 * nb)) continue;
+#pragma unroll
+      for (int c = 0; c < 2; ++c) {
+        const T* src = patch + 2 * nb * C::VEC + tr_off + 16 * c * 8;
+        const V8 dsb = hw::join_v8<T>(hw::lds_read_tr16(src), hw::lds_read_tr16(src + 8 * 8));
+#pragma unroll
+        for (int db = 0; db < C::DV / 32; ++db)
+          dq[db] = hw::mfma32(operand_transposed<T, C::LD>(sK, nb * 32 + 16 * c, db * 32, lane), dsb, dq[db]);
+      }
+    }
+
+    if (more) commit((it + 1) & 1);
+    hw::block_sync();
+  }
+
+  if (my_m < M) {
+    T* o1 = (T*)p.dq.ptr + batch * p.dq.sb + head * p.dq.sh + (int64_t)my_m * p.dq.st;
+#pragma unroll
+    for (int db = 0; db < C::DV / 32; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        int d = db * 32 + 8 * g + 4 * hh;
+        if (d < D) {
+          hw::u32x2 w;
+          w[0] = (uint32_t)hw::bits16<T>(dq[db][4 * g + 0] * p.sm_scale) | ((uint32_t)hw::bits16<T>(dq[db][4 * g + 1] * p.sm_scale) << 16);
+          w[1] = (uint32_t)hw::bits16<T>(dq[db][4 * g + 2] * p.sm_scale) | ((uint32_t)hw::bits16<T>(dq[db][4 * g + 3] * p.sm_scale) << 16);
+          *(hw::u32x2*)(o1 + d) = w;
+        }
+      }
+  }
+}
+
 // ------------------------------------------------------------------------------ launchers ----
 template <class T, bool PW>
 static int launch_dkdv(const BwdParams& p, hipStream_t stream) {
@@ -542,6 +694,48 @@ int run_bwd_dq(const BwdParams& p, bool piecewise, hipStream_t stream) {
     return piecewise ? launch_dq<hw::half_t, true>(p, stream) : launch_dq<hw::half_t, false>(p, stream);
   if (p.dtype == kDtypeBF16)
     return piecewise ? launch_dq<hw::bf16_t, true>(p, stream) : launch_dq<hw::bf16_t, false>(p, stream);
+  return kUnsupported;
+}
+
+template <class T>
+static int launch_dkdv_ds(const BwdParams& p, hipStream_t stream) {
+  dim3 grid(((p.N + 127) / 128) * p.H * p.B, 1, 1);
+  switch (p.D) {
+    case 16: return launch(fa_bwd_dkdv_kernel<T, 16, false, true>, grid, KvCfg<T, 16, false>::LDS_BYTES, stream, p);
+    case 32: return launch(fa_bwd_dkdv_kernel<T, 32, false, true>, grid, KvCfg<T, 32, false>::LDS_BYTES, stream, p);
+    case 64: return launch(fa_bwd_dkdv_kernel<T, 64, false, true>, grid, KvCfg<T, 64, false>::LDS_BYTES, stream, p);
+    case 128: return launch(fa_bwd_dkdv_kernel<T, 128, false, true>, grid, KvCfg<T, 128, false>::LDS_BYTES, stream, p);
+  }
+  return kUnsupported;
+}
+
+template <class T>
+static int launch_dq_from_ds(const BwdParams& p, hipStream_t stream) {
+  dim3 grid(((p.M + 127) / 128) * p.H * p.B, 1, 1);
+  switch (p.D) {
+    case 16: return launch(fa_bwd_dq_from_ds_kernel<T, 16>, grid, QdsCfg<T, 16>::LDS_BYTES, stream, p);
+    case 32: return launch(fa_bwd_dq_from_ds_kernel<T, 32>, grid, QdsCfg<T, 32>::LDS_BYTES, stream, p);
+    case 64: return launch(fa_bwd_dq_from_ds_kernel<T, 64>, grid, QdsCfg<T, 64>::LDS_BYTES, stream, p);
+    case 128: return launch(fa_bwd_dq_from_ds_kernel<T, 128>, grid, QdsCfg<T, 128>::LDS_BYTES, stream, p);
+  }
+  return kUnsupported;
+}
+
+int64_t bwd_ds_workspace_bytes(int B, int H, int M, int N) {
+  return (int64_t)B * H * (4 * (int64_t)((M + 127) / 128)) * (4 * (int64_t)((N + 127) / 128)) * 2048;
+}
+
+int run_bwd_dkdv_ds(const BwdParams& p, hipStream_t stream) {
+  if (p.B <= 0 || p.H <= 0 || p.M <= 0 || p.N <= 0 || p.group <= 0 || !p.ds) return kBadArgument;
+  if (p.dtype == kDtypeF16) return launch_dkdv_ds<hw::half_t>(p, stream);
+  if (p.dtype == kDtypeBF16) return launch_dkdv_ds<hw::bf16_t>(p, stream);
+  return kUnsupported;
+}
+
+int run_bwd_dq_from_ds(const BwdParams& p, hipStream_t stream) {
+  if (p.B <= 0 || p.H <= 0 || p.M <= 0 || p.N <= 0 || p.group <= 0 || !p.ds) return kBadArgument;
+  if (p.dtype == kDtypeF16) return launch_dq_from_ds<hw::half_t>(p, stream);
+  if (p.dtype == kDtypeBF16) return launch_dq_from_ds<hw::bf16_t>(p, stream);
   return kUnsupported;
 }
 

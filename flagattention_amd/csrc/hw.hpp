@@ -90,6 +90,11 @@ FA_DEVICE float shfl_xor(float x, int mask) { return __shfl_xor(x, mask, 64); }
 // Tells the compiler that x has the same value in every lane (kept in a scalar register).
 FA_DEVICE int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
 
+// 16-byte global accesses for data that is written once and read once much later (or read once):
+// marked non-temporal so that they do not displace the tiles the kernel re-reads from the L2.
+FA_DEVICE void store_streaming(void* p, u32x4 v) { __builtin_nontemporal_store(v, (u32x4*)p); }
+FA_DEVICE u32x4 load_streaming(const void* p) { return __builtin_nontemporal_load((const u32x4*)p); }
+
 // Marks a branch body as not speculatable, so that a wavefront-uniform `if` stays a branch instead
 // of being turned into unconditional arithmetic on selected operands.
 FA_DEVICE void keep_branch() { asm volatile("" ::: "memory"); }

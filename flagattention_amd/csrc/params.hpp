@@ -28,6 +28,7 @@ struct BwdParams {
   View4 dq, dk, dv, dq2, dk2;  // written; dk/dv have one slice per *query* head
   const float* lse;            // (B, H, M)
   float* delta;                // (B, H, M) rowsum(O * dO): written by the preprocess, read by the rest
+  void* ds;                    // optional dS workspace: written by the dK/dV kernel, read by dQ-from-dS
   int B, H, M, N, D;
   int group;
   int causal;
@@ -102,6 +103,9 @@ struct PagedParams {
   float* ws; int num_wgs;
 };
 
+int64_t bwd_ds_workspace_bytes(int B, int H, int M, int N);
+int run_bwd_dkdv_ds(const BwdParams& p, hipStream_t stream);
+int run_bwd_dq_from_ds(const BwdParams& p, hipStream_t stream);
 int run_splitkv(const SplitParams& p, hipStream_t stream);
 int run_combine(const CombineParams& p, hipStream_t stream);
 int run_paged(const PagedParams& p, hipStream_t stream);

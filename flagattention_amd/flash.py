@@ -6,6 +6,7 @@ q, k, v only, gradients flowing into the auxiliary outputs are ignored).  The Tr
 replaced by calls into the C-ABI kernel library.
 """
 import math
+import os
 
 import torch
 
@@ -93,13 +94,55 @@ class FlashAttention(torch.autograd.Function):
             # one dK/dV slice per query head; groups are summed afterwards (as flash.py:205-206,250-251)
             dk = torch.empty((B, H, N, D), dtype=k.dtype, device=q.device)
             dv = torch.empty((B, H, N, D), dtype=v.dtype, device=q.device)
-            _abi.fa_bwd_dkdv(lib, q, k, v, do, L, delta, dk, dv, causal, sm_scale)
             dq = torch.empty((B, H, M, D), dtype=q.dtype, device=q.device)
-            _abi.fa_bwd_dq(lib, q, k, v, do, L, delta, dq, causal, sm_scale)
+            heads = ds_heads_per_launch(lib, B, H, group, M, N, D)
+            if heads == 0:
+                _abi.fa_bwd_dkdv(lib, q, k, v, do, L, delta, dk, dv, causal, sm_scale)
+                _abi.fa_bwd_dq(lib, q, k, v, do, L, delta, dq, causal, sm_scale)
+            elif heads >= B * H:
+                ds = _ds_workspace(lib, q.device, B, H, M, N)
+                _abi.fa_bwd_dkdv_ds(lib, q, k, v, do, L, delta, dk, dv, ds, causal, sm_scale)
+                _abi.fa_bwd_dq_from_ds(lib, k, ds, dq, causal, sm_scale)
+            else:
+                # bounded workspace: one batch entry and `heads` query heads at a time
+                heads = min(heads, H)
+                ds = _ds_workspace(lib, q.device, 1, heads, M, N)
+                for b in range(B):
+                    for h0 in range(0, H, heads):
+                        hs, ks = slice(h0, min(H, h0 + heads)), slice(h0 // group, -(-min(H, h0 + heads) // group))
+                        bs = slice(b, b + 1)
+                        _abi.fa_bwd_dkdv_ds(lib, q[bs, hs], k[bs, ks], v[bs, ks], do[bs, hs], L[bs, hs],
+                                            delta[bs, hs], dk[bs, hs], dv[bs, hs], ds, causal, sm_scale)
+                        _abi.fa_bwd_dq_from_ds(lib, k[bs, ks], ds, dq[bs, hs], causal, sm_scale)
             if group > 1:
                 dk = dk.reshape(B, Hk, group, N, D).sum(2)
                 dv = dv.reshape(B, Hk, group, N, D).sum(2)
         return dq, dk, dv, None, None, None, None, None, None
+
+
+# Largest dS workspace the backward may take (MiB); 0 disables the dS path.
+DS_WORKSPACE_LIMIT_MIB = int(os.environ.get("FLAGATTN_DS_WORKSPACE_MIB", "8192"))
+
+
+def ds_heads_per_launch(lib, B, H, group, M, N, D):
+    """How many (batch, head) slices one dK/dV + dQ-from-dS launch pair may cover, 0 = recompute dS
+    in the dQ kernel instead.  Keeping dS costs M * N * 2 bytes per head, written once and read once;
+    it pays when the two recomputed products are expensive (head size 128) and the matrix is big
+    enough for the launches to fill the device."""
+    if D < 128 or M * N < 1024 * 1024 or DS_WORKSPACE_LIMIT_MIB <= 0:
+        return 0
+    per_head = lib.fa_bwd_ds_workspace_mib(1, 1, M, N)
+    fit = DS_WORKSPACE_LIMIT_MIB // per_head
+    if fit >= B * H:
+        return B * H
+    fit = (fit // group) * group  # whole groups of query heads, so that k/v slices line up
+    return fit
+
+
+def _ds_workspace(lib, device, B, H, M, N):
+    mib = lib.fa_bwd_ds_workspace_mib(B, H, M, N)
+    assert mib > 0
+    return torch.empty(mib << 20, dtype=torch.uint8, device=device)
 
 
 def attention(q, k, v, causal=False, sm_scale=None, dropout_p=0.0,

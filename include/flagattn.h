@@ -70,6 +70,23 @@ int fa_bwd_dq(int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v
               const fa_view4* dout, const float* lse, const float* delta, const fa_view4* dq, int B,
               int H, int Hk, int M, int N, int D, int causal, float sm_scale, void* stream);
 
+/* The same backward with dS kept instead of recomputed (no counterpart in the reference, whose
+ * `_bwd_q_kernel`, flash.py:748-909, recomputes the scores, the probabilities and dP): fa_bwd_dkdv_ds
+ * is fa_bwd_dkdv that also leaves dS, rounded to the input dtype, in `ds_workspace`, and
+ * fa_bwd_dq_from_ds computes dq = sm_scale * dS k from it -- one matrix product instead of three,
+ * for one write and one read of a (B, H, M, N) matrix.  The workspace is device memory of at least
+ * fa_bwd_ds_workspace_mib(B, H, M, N) MiB, 16-byte aligned, in a private blocked order; its contents
+ * on entry do not matter.  Both calls must use the same B, H, M, N and causal flag; to bound the
+ * workspace, callers may process slices of the batch or of the heads one after the other. */
+int fa_bwd_ds_workspace_mib(int B, int H, int M, int N);
+int fa_bwd_dkdv_ds(int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v,
+                   const fa_view4* dout, const float* lse, const float* delta, const fa_view4* dk,
+                   const fa_view4* dv, void* ds_workspace, int64_t ds_workspace_bytes, int B, int H,
+                   int Hk, int M, int N, int D, int causal, float sm_scale, void* stream);
+int fa_bwd_dq_from_ds(int dtype, const fa_view4* k, const void* ds_workspace, int64_t ds_workspace_bytes,
+                      const fa_view4* dq, int B, int H, int Hk, int M, int N, int D, int causal,
+                      float sm_scale, void* stream);
+
 /* ------------------------------------------------------------------------- total attention --
  * Replaces `_total_attention_kernel` (src/flag_attn/total.py:50-142; launches flash.py:128-140 and
  * total.py:35-46): total[b,h,n] = sum_m softmax(scores)[m,n], recomputed from q, k and lse. */

@@ -196,6 +196,8 @@ inline int block_x() { return hwsim::bx; }
 inline int block_y() { return hwsim::by; }
 inline int block_z() { return hwsim::bz; }
 inline int grid_x() { return hwsim::gx; }
+inline void store_streaming(void* p, u32x4 v) { *(u32x4*)p = v; }
+inline u32x4 load_streaming(const void* p) { return *(const u32x4*)p; }
 inline int uniform(int x) { return x; }
 inline int grid_z() { return hwsim::gz; }
 inline void block_sync() { hwsim::yield(hwsim::OP_BARRIER); }

@@ -162,3 +162,64 @@ def test_flash_attention_split_kv_entry(causal):
     same = oracle_flash(q, k, v, causal, upcast=False)
     hyp = flag_attn.flash_attention_split_kv(q, k, v, causal)
     check("o", hyp, same, ref)
+
+
+def _grads(q, k, v, do, causal):
+    o = flag_attn.flash_attention(q, k, v, causal)
+    return (o,) + torch.autograd.grad(o, (q, k, v), do)
+
+
+@pytest.mark.parametrize("Hk", [8, 2])
+def test_backward_with_bounded_ds_workspace_matches_unbounded(Hk, monkeypatch):
+    """Head size 128 keeps dS in a workspace for the dQ kernel; with a small limit the backward walks
+    the batch and the heads in slices.  Both must give the very same bits, and the same dQ as the
+    kernel that recomputes dS (limit 0)."""
+    from flagattention_amd import flash as flash_mod
+    q = make((2, 8, 1024, 128), torch.bfloat16, "BTHD", 1.0, 1, grad=True)
+    k = make((2, Hk, 1100, 128), torch.bfloat16, "BTHD", 1.0, 2, grad=True)
+    v = make((2, Hk, 1100, 128), torch.bfloat16, "BTHD", 1.0, 3, grad=True)
+    do = make((2, 8, 1024, 128), torch.bfloat16, "BHTD", 1.0, 4)
+    lib = flash_mod._lib.get()
+    per_head = lib.fa_bwd_ds_workspace_mib(1, 1, 1024, 1100)
+    assert flash_mod.ds_heads_per_launch(lib, 2, 8, 8 // Hk, 1024, 1100, 128) == 16
+    whole = _grads(q, k, v, do, True)
+    monkeypatch.setattr(flash_mod, "DS_WORKSPACE_LIMIT_MIB", 5 * per_head)   # 4 (or 5) heads per launch
+    assert 0 < flash_mod.ds_heads_per_launch(lib, 2, 8, 8 // Hk, 1024, 1100, 128) < 16
+    sliced = _grads(q, k, v, do, True)
+    monkeypatch.setattr(flash_mod, "DS_WORKSPACE_LIMIT_MIB", 0)
+    assert flash_mod.ds_heads_per_launch(lib, 2, 8, 8 // Hk, 1024, 1100, 128) == 0
+    recomputed = _grads(q, k, v, do, True)
+    for a, b, c in zip(whole, sliced, recomputed):
+        assert torch.equal(a, b) and torch.equal(a, c)
+
+
+def test_full_size_backward_paths_agree():
+    """The benchmark's shape (1 x 32 heads x 8192 x 128, causal, bf16) is too large for the fp32
+    oracle over all heads; what does not depend on size: dQ from the stored dS equals dQ from the
+    recomputed dS bit for bit, gradients are linear in dO, and 2 heads are checked against the oracle."""
+    from flagattention_amd import flash as flash_mod
+    q = make((1, 32, 8192, 128), torch.bfloat16, "BHTD", 1.0, 1, grad=True)
+    k = make((1, 32, 8192, 128), torch.bfloat16, "BHTD", 1.0, 2, grad=True)
+    v = make((1, 32, 8192, 128), torch.bfloat16, "BHTD", 1.0, 3, grad=True)
+    do = make((1, 32, 8192, 128), torch.bfloat16, "BHTD", 1.0, 4)
+    stored = _grads(q, k, v, do, True)
+    doubled = _grads(q, k, v, do * 2, True)   # exact in bf16: every product and sum scales by 2
+    for a, b in zip(stored[1:], doubled[1:]):
+        assert torch.equal(a * 2, b)
+    saved = flash_mod.DS_WORKSPACE_LIMIT_MIB
+    try:
+        flash_mod.DS_WORKSPACE_LIMIT_MIB = 0
+        recomputed = _grads(q, k, v, do, True)
+    finally:
+        flash_mod.DS_WORKSPACE_LIMIT_MIB = saved
+    for a, b in zip(stored, recomputed):
+        assert torch.equal(a, b)
+    hs = slice(30, 32)
+    qs, ks, vs = (t[:, hs].detach().requires_grad_() for t in (q, k, v))
+    o_ref = oracle_flash(qs, ks, vs, True, upcast=True)
+    g_ref = torch.autograd.grad(o_ref, (qs, ks, vs), do[:, hs])
+    o_same = oracle_flash(qs, ks, vs, True, upcast=False)
+    g_same = torch.autograd.grad(o_same, (qs, ks, vs), do[:, hs])
+    check("o", stored[0][:, hs], o_same, o_ref)
+    for name, h, s, r in zip(("dq", "dk", "dv"), stored[1:], g_same, g_ref):
+        check(name, h[:, hs], s, r)

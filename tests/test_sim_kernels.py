@@ -83,6 +83,57 @@ def test_flash_forward_backward_total(lib, B, H, Hk, M, N, D, causal, dtype, bth
         assert torch.all(torch.isinf(lse[:, :, : M - N]))
 
 
+DS_CASES = [
+    # B, H, Hk, M, N, D, causal, dtype, bthd
+    (1, 2, 1, 100, 150, 128, True, torch.bfloat16, False),
+    (1, 2, 2, 130, 70, 64, True, torch.float16, True),      # M > N: rows without keys
+    (2, 1, 1, 70, 200, 32, False, torch.bfloat16, True),
+    (1, 1, 1, 257, 129, 16, True, torch.float16, False),    # three query blocks, key tail of one
+]
+
+
+@pytest.mark.parametrize("B,H,Hk,M,N,D,causal,dtype,bthd", DS_CASES)
+def test_flash_backward_with_stored_ds(lib, B, H, Hk, M, N, D, causal, dtype, bthd):
+    """dK/dV kernel that leaves dS in the workspace + dQ computed from it, against the oracle and
+    against the recomputing dQ kernel (the two round dS to the input dtype at the same place)."""
+    q = rnd((B, H, M, D), dtype, bthd).requires_grad_()
+    k = rnd((B, Hk, N, D), dtype, bthd).requires_grad_()
+    v = rnd((B, Hk, N, D), dtype, bthd).requires_grad_()
+    do = rnd((B, H, M, D), dtype, bthd)
+    sc = 1 / math.sqrt(D)
+    qd, kd, vd = q.detach(), k.detach(), v.detach()
+    o = torch.full_like(qd, float("nan"))
+    lse = torch.full((B, H, M), float("nan"))
+    _abi.fa_fwd(lib, qd, kd, vd, o, lse, causal, sc)
+    delta = torch.full((B, H, M), float("nan"))
+    _abi.fa_bwd_delta(lib, o, do, delta)
+    dk = torch.full((B, H, N, D), float("nan"), dtype=dtype)
+    dv = torch.full((B, H, N, D), float("nan"), dtype=dtype)
+    dq = torch.full((B, H, M, D), float("nan"), dtype=dtype)
+    mib = lib.fa_bwd_ds_workspace_mib(B, H, M, N)
+    assert mib > 0
+    ds = torch.full((mib << 19,), float("nan"), dtype=dtype)   # unwritten chunks hold NaN
+    _abi.fa_bwd_dkdv_ds(lib, qd, kd, vd, do, lse, delta, dk, dv, ds, causal, sc)
+    _abi.fa_bwd_dq_from_ds(lib, kd, ds, dq, causal, sc)
+    dk_plain, dv_plain = torch.empty_like(dk), torch.empty_like(dv)
+    dq_plain = torch.empty_like(dq)
+    _abi.fa_bwd_dkdv(lib, qd, kd, vd, do, lse, delta, dk_plain, dv_plain, causal, sc)
+    _abi.fa_bwd_dq(lib, qd, kd, vd, do, lse, delta, dq_plain, causal, sc)
+    assert torch.equal(dk, dk_plain) and torch.equal(dv, dv_plain)
+    assert not torch.isnan(dq).any()
+    g = H // Hk
+    dk, dv = dk.reshape(B, Hk, g, N, D).sum(2), dv.reshape(B, Hk, g, N, D).sum(2)
+    ref = flash_attention(q, k, v, causal, upcast=True)
+    same = flash_attention(q, k, v, causal, upcast=False)
+    g_ref = torch.autograd.grad(ref, (q, k, v), do)
+    g_same = torch.autograd.grad(same, (q, k, v), do)
+    check("dq", dq, g_same[0], g_ref[0])
+    check("dk", dk, g_same[1], g_ref[1])
+    check("dv", dv, g_same[2], g_ref[2])
+    # same products, same rounding of dS; only the summation order over keys inside the MFMA differs
+    assert (dq.float() - dq_plain.float()).abs().max() <= 2e-2 * dq_plain.float().abs().max() + 1e-6
+
+
 PW_CASES = [
     # B, H, M, N, D, w, causal, dtype
     (1, 2, 200, 200, 64, 50, True, torch.bfloat16),
