@@ -75,19 +75,24 @@ struct KvCfg {
   static constexpr int KSTEPS = D / 16;
   static constexpr int LD = DV + 40;  // rows 20 banks apart: 16-byte row reads conflict-free, transposing reads nearly so
   static constexpr int TILE = BM * LD;
-  static constexpr int NTILES = PW ? 3 : 2;  // Q, (Q2), dO
   // register budget: two wavefronts per SIMD (256 registers each) when the accumulators allow it
-  static constexpr int WAVES_PER_SIMD = (D <= 64 && !(PW && D == 64)) ? 2 : 1;
-  static constexpr size_t STAGE_BYTES = NTILES * TILE * sizeof(T) + 2 * BM * sizeof(float);
+  static constexpr int WAVES_PER_SIMD = D <= 64 ? 2 : 1;
+  static constexpr size_t STAGE_BYTES = 2 * TILE * sizeof(T) + 2 * BM * sizeof(float);  // Q, dO, L, delta
   static constexpr size_t LDS_BYTES = 2 * STAGE_BYTES;
 };
 
+// PW (piecewise): the score of (m, n) comes from (q2, k2) when the distance m + pseq - n is >= w and
+// from (q1, k1) otherwise.  The two regimes are two passes over the query tiles -- the near rows
+// with (q1, k1) accumulating dK1, then the far rows with (q2, k2) accumulating dK2 in the same
+// registers -- each masking the entries of the other; dV accumulates over both.
+//
 // DS: also leave dS (rounded to T, as it enters dK += dS^T Q) in the workspace p.ds for
 // fa_bwd_dq_from_ds_kernel, one 2 KB chunk per 32 x 32 block in the order the MFMA result holds it:
 // chunk[c][lane] = 8 elements, queries 16c + 8g + 4(lane / 32) + e at position 4g + e, key lane % 32.
 // Chunks are indexed (batch * H + head, key block, query block); both counts padded to 4.
 template <class T, int D, bool PW, bool DS = false>
 FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (KvCfg<T, D, PW>::WAVES_PER_SIMD)) fa_bwd_dkdv_kernel(BwdParams p) {
+  static_assert(!(PW && DS), "the dS workspace is only defined for plain flash attention");
   using C = KvCfg<T, D, PW>;
   using V8 = typename hw::Elem<T>::v8;
   FA_LDS_DECL(smem);
@@ -100,34 +105,26 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (KvCfg<T, D, PW>::WAVES_PER_SIMD)) fa
   const int M = p.M, N = p.N, pseq = N - M;
   const int n0 = wg.rank * C::BN, nw = n0 + wave * 32, my_n = nw + l32;
 
-  const T* qb = (const T*)p.q.ptr + batch * p.q.sb + head * p.q.sh;
-  const T* q2b = PW ? (const T*)p.q2.ptr + batch * p.q2.sb + head * p.q2.sh : nullptr;
   const T* gb = (const T*)p.dout.ptr + batch * p.dout.sb + head * p.dout.sh;
-  const T* kb = (const T*)p.k.ptr + batch * p.k.sb + hk * p.k.sh;
-  const T* k2b = PW ? (const T*)p.k2.ptr + batch * p.k2.sb + hk * p.k2.sh : nullptr;
   const T* vb = (const T*)p.v.ptr + batch * p.v.sb + hk * p.v.sh;
   const float* lse = p.lse + ((int64_t)batch * p.H + head) * M;
   const float* dlt = p.delta + ((int64_t)batch * p.H + head) * M;
 
-  // K, (K2), V rows of this lane as B operands (k = 16 kk + 8 hh + 0..7)
-  V8 kreg[C::KSTEPS], vreg[C::KSTEPS], k2reg[PW ? C::KSTEPS : 1];
+  // K (of the current regime) and V rows of this lane as B operands (k = 16 kk + 8 hh + 0..7)
+  V8 kreg[C::KSTEPS], vreg[C::KSTEPS];
+  auto load_rows = [&](V8* dst, const T* base, int64_t row_stride) {
 #pragma unroll
-  for (int kk = 0; kk < C::KSTEPS; ++kk) {
-    u32x4 a = {0u, 0u, 0u, 0u}, b = a, c = a;
-    if (my_n < N) {
-      a = *(const u32x4*)(kb + (int64_t)my_n * p.k.st + 16 * kk + 8 * hh);
-      b = *(const u32x4*)(vb + (int64_t)my_n * p.v.st + 16 * kk + 8 * hh);
-      if (PW) c = *(const u32x4*)(k2b + (int64_t)my_n * p.k2.st + 16 * kk + 8 * hh);
+    for (int kk = 0; kk < C::KSTEPS; ++kk) {
+      u32x4 a = {0u, 0u, 0u, 0u};
+      if (my_n < N) a = *(const u32x4*)(base + (int64_t)my_n * row_stride + 16 * kk + 8 * hh);
+      dst[kk] = hw::as_v8<T>(a);
     }
-    kreg[kk] = hw::as_v8<T>(a);
-    vreg[kk] = hw::as_v8<T>(b);
-    if (PW) k2reg[kk] = hw::as_v8<T>(c);
-  }
+  };
+  load_rows(vreg, vb, p.v.st);
 
   // first query tile that can see a key of this block under the causal mask
   int m_lo = 0;
   if (p.causal) m_lo = (imax(0, n0 - pseq) / C::BM) * C::BM;
-  const int n_tiles = m_lo < M ? cdiv(M - m_lo, C::BM) : 0;
 
   if (C::DV != D) {
     T* z = (T*)smem;
@@ -135,14 +132,11 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (KvCfg<T, D, PW>::WAVES_PER_SIMD)) fa
     hw::block_sync();
   }
 
-  f32x16 dk[C::DV / 32], dv[C::DV / 32], dk2[PW ? C::DV / 32 : 1];
+  f32x16 dk[C::DV / 32], dv[C::DV / 32];
 #pragma unroll
   for (int i = 0; i < C::DV / 32; ++i)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) { dk[i][r] = 0.f; dv[i][r] = 0.f; if (PW) dk2[i][r] = 0.f; }
-
-  auto tile_needs_near = [&](int m0) { return !PW || (m0 + pseq - (n0 + C::BN - 1) < p.w); };
-  auto tile_needs_far = [&](int m0) { return PW && (m0 + C::BM - 1 + pseq - n0 >= p.w); };
+    for (int r = 0; r < 16; ++r) { dk[i][r] = 0.f; dv[i][r] = 0.f; }
 
   // dS chunks of this wavefront's key block: one row of the (key block, query block) chunk grid
   T* ds_row = nullptr;
@@ -151,15 +145,15 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (KvCfg<T, D, PW>::WAVES_PER_SIMD)) fa
     ds_row = (T*)p.ds + ((((int64_t)batch * p.H + head) * nkb + (n0 / 32 + wave)) * nqb) * 1024 + lane * 8;
   }
 
-  TileMover<T, C::BM, D> qr, q2r, gr;
-  qr.init(tid, p.q.st);
+  bool far_phase = false;
+  const T* q_src = nullptr;
+  int64_t q_stride = 0;
+  TileMover<T, C::BM, D> qr, gr;
   gr.init(tid, p.dout.st);
-  if (PW) q2r.init(tid, p.q2.st);
   float l_reg = 0.f, d_reg = 0.f;
   auto fetch = [&](int m0) {
     const int rows = M - m0;
-    if (tile_needs_near(m0)) qr.fetch(qb + (int64_t)m0 * p.q.st, rows);
-    if (tile_needs_far(m0)) q2r.fetch(q2b + (int64_t)m0 * p.q2.st, rows);
+    qr.fetch(q_src + (int64_t)m0 * q_stride, rows);
     gr.fetch(gb + (int64_t)m0 * p.dout.st, rows);
     if (tid < C::BM) {
       int m = m0 + tid;
@@ -168,146 +162,143 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (KvCfg<T, D, PW>::WAVES_PER_SIMD)) fa
       d_reg = m < M ? dlt[m] : 0.f;
     }
   };
-  auto commit = [&](int m0, int stage) {
+  auto commit = [&](int stage) {
     unsigned char* base = smem + stage * C::STAGE_BYTES;
     T* s = (T*)base;
-    if (tile_needs_near(m0)) qr.template commit<C::LD>(s);
-    if (tile_needs_far(m0)) q2r.template commit<C::LD>(s + C::TILE);
-    gr.template commit<C::LD>(s + (C::NTILES - 1) * C::TILE);
-    float* f = (float*)(base + C::NTILES * C::TILE * sizeof(T));
+    qr.template commit<C::LD>(s);
+    gr.template commit<C::LD>(s + C::TILE);
+    float* f = (float*)(base + 2 * C::TILE * sizeof(T));
     if (tid < C::BM) { f[tid] = l_reg; f[C::BM + tid] = d_reg; }
   };
 
-  if (n_tiles > 0) { fetch(m_lo); commit(m_lo, 0); }
-  hw::block_sync();
-
   const float c2 = p.sm_scale * kLog2e;
 
-  for (int it = 0; it < n_tiles; ++it) {
-    const int m0 = m_lo + it * C::BM;
-    const bool more = it + 1 < n_tiles;
-    if (more) fetch(m0 + C::BM);
-
-    const unsigned char* base = smem + (it & 1) * C::STAGE_BYTES;
-    const T* sQ = (const T*)base;
-    const T* sQ2 = sQ + C::TILE;
-    const T* sG = sQ + (C::NTILES - 1) * C::TILE;
-    const float* sL = (const float*)(base + C::NTILES * C::TILE * sizeof(T));
-    const float* sDl = sL + C::BM;
-
+  // result block (keys x D): D along lanes, keys along registers
+  auto store_keys = [&](const f32x16* acc, const View4& dst, float scale) {
+    T* base = (T*)dst.ptr + batch * dst.sb + head * dst.sh;
 #pragma unroll
-    for (int sb = 0; sb < C::BM / 32; ++sb) {
-      const int mr0 = m0 + sb * 32;
-      // every (m, n) of this 32 x 32 block is masked: nothing to add
-      if (p.causal && (mr0 + 31 + pseq < nw)) continue;
-      bool near = true, far = false;
-      if (PW) {
-        near = (mr0 + pseq - (nw + 31)) < p.w;
-        far = (mr0 + 31 + pseq - nw) >= p.w;
+    for (int db = 0; db < C::DV / 32; ++db) {
+      const int d = db * 32 + l32;
+      if (d < D) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int n = nw + block_row(r, hh);
+          if (n < N) base[(int64_t)n * dst.st + d] = (T)(acc[db][r] * scale);
+        }
       }
-      f32x16 s, s2, dp;
+    }
+  };
+
+  int stage = 0;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) { s[r] = 0.f; s2[r] = 0.f; dp[r] = 0.f; }
-      if (near) {
+  for (int ph = 0; ph < (PW ? 2 : 1); ++ph) {
+    far_phase = PW && ph == 1;
+    // query tiles [t_begin, t_end) of 64 rows that hold an entry of this regime for some key of the block
+    int t_begin = m_lo / C::BM, t_end = cdiv(M, C::BM);
+    if (PW) {
+      if (far_phase) t_begin = imax(t_begin, imax(0, n0 + p.w - pseq) / C::BM);
+      else t_end = imin(t_end, cdiv(imax(0, imin(M, n0 + C::BN - 1 + p.w - pseq)), C::BM));
+    }
+    if (t_begin < t_end) {
+      q_src = (const T*)(far_phase ? p.q2.ptr : p.q.ptr) + batch * (far_phase ? p.q2.sb : p.q.sb) +
+              head * (far_phase ? p.q2.sh : p.q.sh);
+      q_stride = far_phase ? p.q2.st : p.q.st;
+      qr.init(tid, q_stride);
+      if (far_phase) load_rows(kreg, (const T*)p.k2.ptr + batch * p.k2.sb + hk * p.k2.sh, p.k2.st);
+      else load_rows(kreg, (const T*)p.k.ptr + batch * p.k.sb + hk * p.k.sh, p.k.st);
+      fetch(t_begin * C::BM);
+      commit(stage);
+      hw::block_sync();
+    }
+
+    for (int it = t_begin; it < t_end; ++it) {
+      const int m0 = it * C::BM;
+      const bool more = it + 1 < t_end;
+      if (more) fetch(m0 + C::BM);
+
+      const unsigned char* base = smem + stage * C::STAGE_BYTES;
+      const T* sQ = (const T*)base;
+      const T* sG = sQ + C::TILE;
+      const float* sL = (const float*)(base + 2 * C::TILE * sizeof(T));
+      const float* sDl = sL + C::BM;
+
+#pragma unroll
+      for (int sb = 0; sb < C::BM / 32; ++sb) {
+        const int mr0 = m0 + sb * 32;
+        // every (m, n) of this 32 x 32 block is masked, or belongs to the other regime: nothing to add
+        if (p.causal && (mr0 + 31 + pseq < nw)) continue;
+        if (PW && (far_phase ? (mr0 + 31 + pseq - nw < p.w) : (mr0 + pseq - (nw + 31) >= p.w))) continue;
+        f32x16 s, dp;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
 #pragma unroll
         for (int kk = 0; kk < C::KSTEPS; ++kk)
           s = hw::mfma32(operand_rowmajor<T, C::LD>(sQ, sb * 32, 16 * kk, lane), kreg[kk], s);
-      }
-      if (PW && far) {
 #pragma unroll
         for (int kk = 0; kk < C::KSTEPS; ++kk)
-          s2 = hw::mfma32(operand_rowmajor<T, C::LD>(sQ2, sb * 32, 16 * kk, lane), k2reg[kk], s2);
-      }
-#pragma unroll
-      for (int kk = 0; kk < C::KSTEPS; ++kk)
-        dp = hw::mfma32(operand_rowmajor<T, C::LD>(sG, sb * 32, 16 * kk, lane), vreg[kk], dp);
-      if (!PW) hw::sched_prefetched_operands<2 * C::KSTEPS, (C::KSTEPS >= 8 ? 8 : 2)>();
+          dp = hw::mfma32(operand_rowmajor<T, C::LD>(sG, sb * 32, 16 * kk, lane), vreg[kk], dp);
+        hw::sched_prefetched_operands<2 * C::KSTEPS, (C::KSTEPS >= 8 ? 8 : 2)>();
 
-      const bool need_mask = p.causal && (mr0 + pseq < nw + 31);
-      // L * log2e and delta of this lane's 16 query rows: rows 8g + 4h + 0..3 are contiguous
-      hw::f32x4 lrow[4], drow[4];
+        bool need_mask = p.causal && (mr0 + pseq < nw + 31);
+        if (PW) need_mask = need_mask || (far_phase ? (mr0 + pseq - (nw + 31) < p.w) : (mr0 + 31 + pseq - nw >= p.w));
+        // L * log2e and delta of this lane's 16 query rows: rows 8g + 4h + 0..3 are contiguous
+        hw::f32x4 lrow[4], drow[4];
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        lrow[g] = *(const hw::f32x4*)(sL + sb * 32 + 8 * g + 4 * hh);
-        drow[g] = *(const hw::f32x4*)(sDl + sb * 32 + 8 * g + 4 * hh);
-      }
-      f32x16 pr, ds, ds2;
-      if (PW || need_mask) {
+        for (int g = 0; g < 4; ++g) {
+          lrow[g] = *(const hw::f32x4*)(sL + sb * 32 + 8 * g + 4 * hh);
+          drow[g] = *(const hw::f32x4*)(sDl + sb * 32 + 8 * g + 4 * hh);
+        }
+        f32x16 pr, ds;
+        if (need_mask) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int m = mr0 + block_row(r, hh);
-          float sv = s[r];
-          bool is_far = false;
-          if (PW) {
-            is_far = (m + pseq - my_n) >= p.w;
-            sv = is_far ? s2[r] : s[r];
+          for (int r = 0; r < 16; ++r) {
+            const int m = mr0 + block_row(r, hh);
+            bool keep = !p.causal || (m + pseq >= my_n);
+            if (PW) keep = keep && ((m + pseq - my_n >= p.w) == far_phase);
+            float pv = hw::exp2_fast(fmaf(s[r], c2, -lrow[r >> 2][r & 3]));
+            pv = keep ? pv : 0.f;
+            pr[r] = pv;
+            ds[r] = pv * (dp[r] - drow[r >> 2][r & 3]);
           }
-          float pv = hw::exp2_fast(fmaf(sv, c2, -lrow[r >> 2][r & 3]));
-          if (need_mask) pv = (m + pseq >= my_n) ? pv : 0.f;
-          float dsv = pv * (dp[r] - drow[r >> 2][r & 3]);
-          pr[r] = pv;
-          if (PW) {
-            ds[r] = is_far ? 0.f : dsv;
-            ds2[r] = is_far ? dsv : 0.f;
-          } else {
-            ds[r] = dsv;
+        } else {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const float pv = hw::exp2_fast(fmaf(s[r], c2, -lrow[r >> 2][r & 3]));
+            pr[r] = pv;
+            ds[r] = pv * (dp[r] - drow[r >> 2][r & 3]);
           }
         }
-      } else {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const float pv = hw::exp2_fast(fmaf(s[r], c2, -lrow[r >> 2][r & 3]));
-          pr[r] = pv;
-          ds[r] = pv * (dp[r] - drow[r >> 2][r & 3]);
-        }
-      }
+        for (int c = 0; c < 2; ++c) {
+          V8 pa = pack_half_block<T>(pr, c);
 #pragma unroll
-      for (int c = 0; c < 2; ++c) {
-        V8 pa = pack_half_block<T>(pr, c);
-#pragma unroll
-        for (int db = 0; db < C::DV / 32; ++db)
-          dv[db] = hw::mfma32(pa, operand_transposed<T, C::LD>(sG, sb * 32 + 16 * c, db * 32, lane), dv[db]);
-        if (near) {
+          for (int db = 0; db < C::DV / 32; ++db)
+            dv[db] = hw::mfma32(pa, operand_transposed<T, C::LD>(sG, sb * 32 + 16 * c, db * 32, lane), dv[db]);
           V8 da = pack_half_block<T>(ds, c);
           if (DS) hw::store_streaming(ds_row + (int64_t)(mr0 / 32) * 1024 + c * 512, __builtin_bit_cast(u32x4, da));
 #pragma unroll
           for (int db = 0; db < C::DV / 32; ++db)
             dk[db] = hw::mfma32(da, operand_transposed<T, C::LD>(sQ, sb * 32 + 16 * c, db * 32, lane), dk[db]);
         }
-        if (PW && far) {
-          V8 da2 = pack_half_block<T>(ds2, c);
-#pragma unroll
-          for (int db = 0; db < C::DV / 32; ++db)
-            dk2[db] = hw::mfma32(da2, operand_transposed<T, C::LD>(sQ2, sb * 32 + 16 * c, db * 32, lane), dk2[db]);
-        }
+        // each of these products takes an operand made of two transposing reads
+        hw::sched_prefetched_operands<4 * (C::DV / 32), (C::DV >= 128 ? 5 : 1), 2>();
       }
-      // each of these products takes an operand made of two transposing reads
-      if (!PW) hw::sched_prefetched_operands<4 * (C::DV / 32), (C::DV >= 128 ? 5 : 1), 2>();
+
+      if (more) commit(stage ^ 1);
+      hw::block_sync();
+      stage ^= 1;
     }
 
-    if (more) commit(m0 + C::BM, (it + 1) & 1);
-    hw::block_sync();
-  }
-
-  // ---- store: result block (keys x D) has D along lanes, keys along registers ----
-  T* dkb = (T*)p.dk.ptr + batch * p.dk.sb + head * p.dk.sh;
-  T* dvb = (T*)p.dv.ptr + batch * p.dv.sb + head * p.dv.sh;
-  T* dk2b = PW ? (T*)p.dk2.ptr + batch * p.dk2.sb + head * p.dk2.sh : nullptr;
+    // this regime's dK is complete
+    store_keys(dk, (PW && far_phase) ? p.dk2 : p.dk, p.sm_scale);
+    if (PW && !far_phase) {
 #pragma unroll
-  for (int db = 0; db < C::DV / 32; ++db) {
-    const int d = db * 32 + l32;
-    if (d < D) {
+      for (int i = 0; i < C::DV / 32; ++i)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int n = nw + block_row(r, hh);
-        if (n < N) {
-          dkb[(int64_t)n * p.dk.st + d] = (T)(dk[db][r] * p.sm_scale);
-          dvb[(int64_t)n * p.dv.st + d] = (T)dv[db][r];
-          if (PW) dk2b[(int64_t)n * p.dk2.st + d] = (T)(dk2[db][r] * p.sm_scale);
-        }
-      }
+        for (int r = 0; r < 16; ++r) dk[i][r] = 0.f;
     }
   }
+  store_keys(dv, p.dv, 1.f);
 }
 
 // ----------------------------------------------------------------------------------- dQ ----
@@ -319,12 +310,13 @@ struct QCfg {
   static constexpr int KSTEPS = D / 16;
   static constexpr int LD = DV + 40;  // rows 20 banks apart: 16-byte row reads conflict-free, transposing reads nearly so
   static constexpr int TILE = BN * LD;
-  static constexpr int NTILES = PW ? 3 : 2;  // K, (K2), V
-  static constexpr int WAVES_PER_SIMD = (PW && D == 128) ? 1 : 2;
-  static constexpr size_t STAGE_BYTES = NTILES * TILE * sizeof(T);
+  static constexpr int WAVES_PER_SIMD = (PW && D == 128) ? 1 : 2;  // the piecewise bookkeeping does not fit 256 registers at 128
+  static constexpr size_t STAGE_BYTES = 2 * TILE * sizeof(T);  // K, V
   static constexpr size_t LDS_BYTES = 2 * STAGE_BYTES;
 };
 
+// PW: two passes over the key tiles, as in the forward kernel -- the far keys with (q2, k2)
+// accumulating dQ2, then the near keys with (q1, k1) accumulating dQ1 in the same registers.
 template <class T, int D, bool PW>
 FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (QCfg<T, D, PW>::WAVES_PER_SIMD)) fa_bwd_dq_kernel(BwdParams p) {
   using C = QCfg<T, D, PW>;
@@ -341,26 +333,20 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (QCfg<T, D, PW>::WAVES_PER_SIMD)) fa_
   const int M = p.M, N = p.N, pseq = N - M;
   const int m0 = mb * C::BM, mw = m0 + wave * 32, my_m = mw + l32;
 
-  const T* qb = (const T*)p.q.ptr + batch * p.q.sb + head * p.q.sh;
-  const T* q2b = PW ? (const T*)p.q2.ptr + batch * p.q2.sb + head * p.q2.sh : nullptr;
   const T* gb = (const T*)p.dout.ptr + batch * p.dout.sb + head * p.dout.sh;
-  const T* kb = (const T*)p.k.ptr + batch * p.k.sb + hk * p.k.sh;
-  const T* k2b = PW ? (const T*)p.k2.ptr + batch * p.k2.sb + hk * p.k2.sh : nullptr;
   const T* vb = (const T*)p.v.ptr + batch * p.v.sb + hk * p.v.sh;
 
-  V8 qreg[C::KSTEPS], greg[C::KSTEPS], q2reg[PW ? C::KSTEPS : 1];
+  // Q (of the current regime) and dO rows of this lane as B operands
+  V8 qreg[C::KSTEPS], greg[C::KSTEPS];
+  auto load_rows = [&](V8* dst, const T* base, int64_t row_stride) {
 #pragma unroll
-  for (int kk = 0; kk < C::KSTEPS; ++kk) {
-    u32x4 a = {0u, 0u, 0u, 0u}, b = a, c = a;
-    if (my_m < M) {
-      a = *(const u32x4*)(qb + (int64_t)my_m * p.q.st + 16 * kk + 8 * hh);
-      b = *(const u32x4*)(gb + (int64_t)my_m * p.dout.st + 16 * kk + 8 * hh);
-      if (PW) c = *(const u32x4*)(q2b + (int64_t)my_m * p.q2.st + 16 * kk + 8 * hh);
+    for (int kk = 0; kk < C::KSTEPS; ++kk) {
+      u32x4 a = {0u, 0u, 0u, 0u};
+      if (my_m < M) a = *(const u32x4*)(base + (int64_t)my_m * row_stride + 16 * kk + 8 * hh);
+      dst[kk] = hw::as_v8<T>(a);
     }
-    qreg[kk] = hw::as_v8<T>(a);
-    greg[kk] = hw::as_v8<T>(b);
-    if (PW) q2reg[kk] = hw::as_v8<T>(c);
-  }
+  };
+  load_rows(greg, gb, p.dout.st);
   // rows past M get L = +inf, hence P = 0
   const int64_t row_off = ((int64_t)batch * p.H + head) * M + my_m;
   const float l_row = my_m < M ? p.lse[row_off] * kLog2e : __builtin_inff();
@@ -375,145 +361,138 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (QCfg<T, D, PW>::WAVES_PER_SIMD)) fa_
     hw::block_sync();
   }
 
-  f32x16 dq[C::DV / 32], dq2[PW ? C::DV / 32 : 1];
+  f32x16 dq[C::DV / 32];
 #pragma unroll
   for (int i = 0; i < C::DV / 32; ++i)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) { dq[i][r] = 0.f; if (PW) dq2[i][r] = 0.f; }
+    for (int r = 0; r < 16; ++r) dq[i][r] = 0.f;
 
-  auto tile_needs_near = [&](int n0) { return !PW || (m0 + pseq - (n0 + C::BN - 1) < p.w); };
-  auto tile_needs_far = [&](int n0) { return PW && (m0 + C::BM - 1 + pseq - n0 >= p.w); };
-
-  TileMover<T, C::BN, D> kr, k2r, vr;
-  kr.init(tid, p.k.st);
+  bool far_phase = false;
+  const T* k_src = nullptr;
+  int64_t k_stride = 0;
+  TileMover<T, C::BN, D> kr, vr;
   vr.init(tid, p.v.st);
-  if (PW) k2r.init(tid, p.k2.st);
   auto fetch = [&](int n0) {
     const int rows = N - n0;
-    if (tile_needs_near(n0)) kr.fetch(kb + (int64_t)n0 * p.k.st, rows);
-    if (tile_needs_far(n0)) k2r.fetch(k2b + (int64_t)n0 * p.k2.st, rows);
+    kr.fetch(k_src + (int64_t)n0 * k_stride, rows);
     vr.fetch(vb + (int64_t)n0 * p.v.st, rows);
   };
-  auto commit = [&](int n0, int stage) {
+  auto commit = [&](int stage) {
     T* s = (T*)(smem + stage * C::STAGE_BYTES);
-    if (tile_needs_near(n0)) kr.template commit<C::LD>(s);
-    if (tile_needs_far(n0)) k2r.template commit<C::LD>(s + C::TILE);
-    vr.template commit<C::LD>(s + (C::NTILES - 1) * C::TILE);
+    kr.template commit<C::LD>(s);
+    vr.template commit<C::LD>(s + C::TILE);
   };
-
-  if (n_tiles > 0) { fetch(0); commit(0, 0); }
-  hw::block_sync();
 
   const float c2 = p.sm_scale * kLog2e;
 
-  for (int it = 0; it < n_tiles; ++it) {
-    const int n0 = it * C::BN;
-    const bool more = it + 1 < n_tiles;
-    if (more) fetch(n0 + C::BN);
-
-    const T* sK = (const T*)(smem + (it & 1) * C::STAGE_BYTES);
-    const T* sK2 = sK + C::TILE;
-    const T* sV = sK + (C::NTILES - 1) * C::TILE;
-
+  // dQ^T blocks: lane owns one query row, registers run along D
+  auto store_rows = [&](const View4& dst) {
+    if (my_m < M) {
+      T* o1 = (T*)dst.ptr + batch * dst.sb + head * dst.sh + (int64_t)my_m * dst.st;
 #pragma unroll
-    for (int nb = 0; nb < C::BN / 32; ++nb) {
-      const int nlo = n0 + nb * 32;
-      if (p.causal && (mw + 31 + pseq < nlo)) continue;  // block fully masked for this wavefront
-      bool near = true, far = false;
-      if (PW) {
-        near = (mw + pseq - (nlo + 31)) < p.w;
-        far = (mw + 31 + pseq - nlo) >= p.w;
+      for (int db = 0; db < C::DV / 32; ++db)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          int d = db * 32 + 8 * g + 4 * hh;
+          if (d < D) {
+            hw::u32x2 w;
+            w[0] = (uint32_t)hw::bits16<T>(dq[db][4 * g + 0] * p.sm_scale) | ((uint32_t)hw::bits16<T>(dq[db][4 * g + 1] * p.sm_scale) << 16);
+            w[1] = (uint32_t)hw::bits16<T>(dq[db][4 * g + 2] * p.sm_scale) | ((uint32_t)hw::bits16<T>(dq[db][4 * g + 3] * p.sm_scale) << 16);
+            *(hw::u32x2*)(o1 + d) = w;
+          }
+        }
+    }
+  };
+
+  int stage = 0;
+#pragma unroll
+  for (int ph = 0; ph < (PW ? 2 : 1); ++ph) {
+    far_phase = PW && ph == 0;
+    int t_begin = 0, t_end = n_tiles;
+    if (PW) {
+      if (far_phase) {
+        const int far_hi = imin(hi, m0 + C::BM + pseq - p.w);
+        t_end = far_hi > 0 ? cdiv(far_hi, C::BN) : 0;
+      } else {
+        t_begin = imax(0, m0 + pseq - p.w + 1) / C::BN;
       }
-      f32x16 s, s2, dp;
+    }
+    if (t_begin < t_end) {
+      k_src = (const T*)(far_phase ? p.k2.ptr : p.k.ptr) + batch * (far_phase ? p.k2.sb : p.k.sb) +
+              hk * (far_phase ? p.k2.sh : p.k.sh);
+      k_stride = far_phase ? p.k2.st : p.k.st;
+      kr.init(tid, k_stride);
+      if (far_phase) load_rows(qreg, (const T*)p.q2.ptr + batch * p.q2.sb + head * p.q2.sh, p.q2.st);
+      else load_rows(qreg, (const T*)p.q.ptr + batch * p.q.sb + head * p.q.sh, p.q.st);
+      fetch(t_begin * C::BN);
+      commit(stage);
+      hw::block_sync();
+    }
+
+    for (int it = t_begin; it < t_end; ++it) {
+      const int n0 = it * C::BN;
+      const bool more = it + 1 < t_end;
+      if (more) fetch(n0 + C::BN);
+
+      const T* sK = (const T*)(smem + stage * C::STAGE_BYTES);
+      const T* sV = sK + C::TILE;
+
 #pragma unroll
-      for (int r = 0; r < 16; ++r) { s[r] = 0.f; s2[r] = 0.f; dp[r] = 0.f; }
-      if (near) {
+      for (int nb = 0; nb < C::BN / 32; ++nb) {
+        const int nlo = n0 + nb * 32;
+        if (p.causal && (mw + 31 + pseq < nlo)) continue;  // block fully masked for this wavefront
+        if (PW && (far_phase ? (mw + 31 + pseq - nlo < p.w) : (mw + pseq - (nlo + 31) >= p.w))) continue;
+        f32x16 s, dp;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
 #pragma unroll
         for (int kk = 0; kk < C::KSTEPS; ++kk)
           s = hw::mfma32(operand_rowmajor<T, C::LD>(sK, nb * 32, 16 * kk, lane), qreg[kk], s);
-      }
-      if (PW && far) {
 #pragma unroll
         for (int kk = 0; kk < C::KSTEPS; ++kk)
-          s2 = hw::mfma32(operand_rowmajor<T, C::LD>(sK2, nb * 32, 16 * kk, lane), q2reg[kk], s2);
-      }
-#pragma unroll
-      for (int kk = 0; kk < C::KSTEPS; ++kk)
-        dp = hw::mfma32(operand_rowmajor<T, C::LD>(sV, nb * 32, 16 * kk, lane), greg[kk], dp);
-      if (!PW) hw::sched_prefetched_operands<2 * C::KSTEPS, (C::KSTEPS >= 4 ? 4 : 2)>();
+          dp = hw::mfma32(operand_rowmajor<T, C::LD>(sV, nb * 32, 16 * kk, lane), greg[kk], dp);
+        hw::sched_prefetched_operands<2 * C::KSTEPS, (C::KSTEPS >= 4 ? 4 : 2)>();
 
-      const bool need_mask = (nlo + 32 > N) || (p.causal && (nlo + 31 > pseq + mw));
-      f32x16 ds, ds2;
-      if (PW || need_mask) {
+        bool need_mask = (nlo + 32 > N) || (p.causal && (nlo + 31 > pseq + mw));
+        if (PW) need_mask = need_mask || (far_phase ? (mw + pseq - (nlo + 31) < p.w) : (mw + 31 + pseq - nlo >= p.w));
+        f32x16 ds;
+        if (need_mask) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int n = nlo + block_row(r, hh);
-          float sv = s[r];
-          bool is_far = false;
-          if (PW) {
-            is_far = (my_m + pseq - n) >= p.w;
-            sv = is_far ? s2[r] : s[r];
+          for (int r = 0; r < 16; ++r) {
+            const int n = nlo + block_row(r, hh);
+            bool keep = (n < N) && (!p.causal || (my_m + pseq >= n));
+            if (PW) keep = keep && ((my_m + pseq - n >= p.w) == far_phase);
+            float pv = hw::exp2_fast(fmaf(s[r], c2, -l_row));
+            pv = keep ? pv : 0.f;
+            ds[r] = pv * (dp[r] - d_row);
           }
-          float pv = hw::exp2_fast(fmaf(sv, c2, -l_row));
-          if (need_mask) pv = ((n < N) && (!p.causal || (my_m + pseq >= n))) ? pv : 0.f;
-          float dsv = pv * (dp[r] - d_row);
-          if (PW) {
-            ds[r] = is_far ? 0.f : dsv;
-            ds2[r] = is_far ? dsv : 0.f;
-          } else {
-            ds[r] = dsv;
-          }
+        } else {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) ds[r] = hw::exp2_fast(fmaf(s[r], c2, -l_row)) * (dp[r] - d_row);
         }
-      } else {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) ds[r] = hw::exp2_fast(fmaf(s[r], c2, -l_row)) * (dp[r] - d_row);
-      }
-#pragma unroll
-      for (int c = 0; c < 2; ++c) {
-        if (near) {
+        for (int c = 0; c < 2; ++c) {
           V8 db_ = pack_half_block<T>(ds, c);
 #pragma unroll
           for (int db = 0; db < C::DV / 32; ++db)
             dq[db] = hw::mfma32(operand_transposed<T, C::LD>(sK, nb * 32 + 16 * c, db * 32, lane), db_, dq[db]);
         }
-        if (PW && far) {
-          V8 db2 = pack_half_block<T>(ds2, c);
-#pragma unroll
-          for (int db = 0; db < C::DV / 32; ++db)
-            dq2[db] = hw::mfma32(operand_transposed<T, C::LD>(sK2, nb * 32 + 16 * c, db * 32, lane), db2, dq2[db]);
-        }
       }
+
+      if (more) commit(stage ^ 1);
+      hw::block_sync();
+      stage ^= 1;
     }
 
-    if (more) commit(n0 + C::BN, (it + 1) & 1);
-    hw::block_sync();
-  }
-
-  // ---- store dQ^T blocks: lane owns one query row, registers run along D ----
-  if (my_m < M) {
-    T* o1 = (T*)p.dq.ptr + batch * p.dq.sb + head * p.dq.sh + (int64_t)my_m * p.dq.st;
-    T* o2 = PW ? (T*)p.dq2.ptr + batch * p.dq2.sb + head * p.dq2.sh + (int64_t)my_m * p.dq2.st : nullptr;
+    store_rows((PW && far_phase) ? p.dq2 : p.dq);
+    if (PW && far_phase) {
 #pragma unroll
-    for (int db = 0; db < C::DV / 32; ++db)
+      for (int i = 0; i < C::DV / 32; ++i)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        int d = db * 32 + 8 * g + 4 * hh;
-        if (d < D) {
-          hw::u32x2 w;
-          w[0] = (uint32_t)hw::bits16<T>(dq[db][4 * g + 0] * p.sm_scale) | ((uint32_t)hw::bits16<T>(dq[db][4 * g + 1] * p.sm_scale) << 16);
-          w[1] = (uint32_t)hw::bits16<T>(dq[db][4 * g + 2] * p.sm_scale) | ((uint32_t)hw::bits16<T>(dq[db][4 * g + 3] * p.sm_scale) << 16);
-          *(hw::u32x2*)(o1 + d) = w;
-          if (PW) {
-            hw::u32x2 w2;
-            w2[0] = (uint32_t)hw::bits16<T>(dq2[db][4 * g + 0] * p.sm_scale) | ((uint32_t)hw::bits16<T>(dq2[db][4 * g + 1] * p.sm_scale) << 16);
-            w2[1] = (uint32_t)hw::bits16<T>(dq2[db][4 * g + 2] * p.sm_scale) | ((uint32_t)hw::bits16<T>(dq2[db][4 * g + 3] * p.sm_scale) << 16);
-            *(hw::u32x2*)(o2 + d) = w2;
-          }
-        }
-      }
+        for (int r = 0; r < 16; ++r) dq[i][r] = 0.f;
+    }
   }
 }
-
 
 // --------------------------------------------------------------------------- dQ from dS ----
 // dQ = scale * dS K with dS read back from the workspace the dK/dV kernel left (see there for the

@@ -24,11 +24,11 @@ struct FwdCfg {
   static constexpr int BM = 128, BN = 64;
   static constexpr int DV = D < 32 ? 32 : D;  // value/output width rounded up to one MFMA block
   static constexpr int KSTEPS = D / 16;
-  static constexpr int WAVES_PER_SIMD = (PW && D == 128) ? 1 : 2;  // register budget per wavefront
+  static constexpr int WAVES_PER_SIMD = 2;  // register budget per wavefront
   static constexpr int K_LD = D + 8;    // 16 B of padding: conflict-free 16-byte row reads
   static constexpr int V_LD = DV + 32;  // 64 B of padding: the 4 rows of a transposing read fall in disjoint banks
   static constexpr int K_TILE = BN * K_LD, V_TILE = BN * V_LD;
-  static constexpr int STAGE = (PW ? 2 : 1) * K_TILE + V_TILE;  // elements per pipeline stage
+  static constexpr int STAGE = K_TILE + V_TILE;  // elements per pipeline stage
   static constexpr size_t LDS_BYTES = 2 * STAGE * sizeof(T);
 };
 
@@ -54,18 +54,16 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (FwdCfg<T, D, PW>::WAVES_PER_SIMD)) f
   const T* q2b = PW ? (const T*)p.q2.ptr + batch * p.q2.sb + head * p.q2.sh : nullptr;
   const T* k2b = PW ? (const T*)p.k2.ptr + batch * p.k2.sb + hk * p.k2.sh : nullptr;
 
-  // ---- Q (and Q2) rows of this lane as B operands: k = 16 * kk + 8 * hh + 0..7 ----
-  V8 qreg[C::KSTEPS], q2reg[PW ? C::KSTEPS : 1];
+  // ---- Q rows of this lane as B operands: k = 16 * kk + 8 * hh + 0..7 ----
+  V8 qreg[C::KSTEPS];
+  auto load_q = [&](const T* base, int64_t row_stride) {
 #pragma unroll
-  for (int kk = 0; kk < C::KSTEPS; ++kk) {
-    u32x4 z = {0u, 0u, 0u, 0u}, z2 = {0u, 0u, 0u, 0u};
-    if (my_m < M) {
-      z = *(const u32x4*)(qb + (int64_t)my_m * p.q.st + 16 * kk + 8 * hh);
-      if (PW) z2 = *(const u32x4*)(q2b + (int64_t)my_m * p.q2.st + 16 * kk + 8 * hh);
+    for (int kk = 0; kk < C::KSTEPS; ++kk) {
+      u32x4 z = {0u, 0u, 0u, 0u};
+      if (my_m < M) z = *(const u32x4*)(base + (int64_t)my_m * row_stride + 16 * kk + 8 * hh);
+      qreg[kk] = hw::as_v8<T>(z);
     }
-    qreg[kk] = hw::as_v8<T>(z);
-    if (PW) q2reg[kk] = hw::as_v8<T>(z2);
-  }
+  };
 
   // ---- key range of this workgroup ----
   int hi = N;
@@ -86,91 +84,54 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (FwdCfg<T, D, PW>::WAVES_PER_SIMD)) f
 #pragma unroll
     for (int r = 0; r < 16; ++r) oacc[i][r] = 0.f;
 
-  // Which key tiles need which (q, k) pair: pair 2 serves distance >= w, pair 1 distance < w.
-  // Over the workgroup's rows and a tile's keys the distance m + pseq - n spans
-  //   [m0 + pseq - (n0 + BN - 1), m0 + BM - 1 + pseq - n0].
-  auto tile_needs_near = [&](int n0) { return !PW || (m0 + pseq - (n0 + C::BN - 1) < p.w); };
-  auto tile_needs_far = [&](int n0) { return PW && (m0 + C::BM - 1 + pseq - n0 >= p.w); };
-
-  TileMover<T, C::BN, D> kr, vr, k2r;
-  kr.init(tid, p.k.st);
+  // Piecewise: the score of (m, n) comes from (q2, k2) when the distance m + pseq - n is >= w and
+  // from (q1, k1) otherwise.  The two regimes are two passes of the same loop -- first the keys far
+  // from this workgroup's rows with (q2, k2), then the near ones with (q1, k1) -- each masking the
+  // entries that belong to the other; the online softmax does not care that a key tile crossed by
+  // the threshold is visited twice.  So the variant needs no more registers or LDS than plain flash.
+  bool far_phase = false;
+  const T* k_src = kb;
+  int64_t k_stride = p.k.st;
+  TileMover<T, C::BN, D> kr, vr;
   vr.init(tid, p.v.st);
-  if (PW) k2r.init(tid, p.k2.st);
   auto fetch = [&](int n0) {
     const int rows = N - n0;
-    if (tile_needs_near(n0)) kr.fetch(kb + (int64_t)n0 * p.k.st, rows);
-    if (tile_needs_far(n0)) k2r.fetch(k2b + (int64_t)n0 * p.k2.st, rows);
+    kr.fetch(k_src + (int64_t)n0 * k_stride, rows);
     vr.fetch(vb + (int64_t)n0 * p.v.st, rows);
   };
-  auto commit = [&](int n0, int stage) {
+  auto commit = [&](int stage) {
     T* s = lds + stage * C::STAGE;
-    if (tile_needs_near(n0)) kr.template commit<C::K_LD>(s);
-    if (tile_needs_far(n0)) k2r.template commit<C::K_LD>(s + C::K_TILE);
-    vr.template commit<C::V_LD>(s + (PW ? 2 : 1) * C::K_TILE);
+    kr.template commit<C::K_LD>(s);
+    vr.template commit<C::V_LD>(s + C::K_TILE);
   };
-
-  if (n_tiles > 0) {
-    fetch(0);
-    commit(0, 0);
-  }
-  hw::block_sync();
 
   const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
   // One key tile; the LDS stage is a compile-time constant so that every operand address is a fixed
   // offset from one per-lane base.
-  auto step = [&](int it, int kStage) {
+  auto step = [&](int it, int t_end, int kStage) {
     const int n0 = it * C::BN;
-    const bool more = it + 1 < n_tiles;
+    const bool more = it + 1 < t_end;
     if (more) fetch(n0 + C::BN);
 
     const T* sK = lds + kStage * C::STAGE;
-    const T* sK2 = sK + C::K_TILE;
-    const T* sV = sK + (PW ? 2 : 1) * C::K_TILE;
+    const T* sV = sK + C::K_TILE;
 
     // ---- S^T = K Q^T : BN/32 blocks of (32 keys x 32 queries) ----
     f32x16 s[C::BN / 32];
 #pragma unroll
     for (int nb = 0; nb < C::BN / 32; ++nb) {
-      const int nlo = n0 + nb * 32;
-      if (!PW) {
-        f32x16 a1 = zero16;
+      f32x16 a1 = zero16;
 #pragma unroll
-        for (int kk = 0; kk < C::KSTEPS; ++kk)
-          a1 = hw::mfma32(operand_rowmajor<T, C::K_LD>(sK, nb * 32, 16 * kk, lane), qreg[kk], a1);
-        s[nb] = a1;
-      } else {
-        // wavefront-uniform: distances over this 32 x 32 block
-        const bool near = (mw + pseq - (nlo + 31)) < p.w;
-        const bool far = (mw + 31 + pseq - nlo) >= p.w;
-        f32x16 a1 = zero16, a2 = zero16;
-        if (near) {
-#pragma unroll
-          for (int kk = 0; kk < C::KSTEPS; ++kk)
-            a1 = hw::mfma32(operand_rowmajor<T, C::K_LD>(sK, nb * 32, 16 * kk, lane), qreg[kk], a1);
-        }
-        if (far) {
-#pragma unroll
-          for (int kk = 0; kk < C::KSTEPS; ++kk)
-            a2 = hw::mfma32(operand_rowmajor<T, C::K_LD>(sK2, nb * 32, 16 * kk, lane), q2reg[kk], a2);
-        }
-        if (far && near) {
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            int n = nlo + block_row(r, hh);
-            a1[r] = (my_m + pseq - n >= p.w) ? a2[r] : a1[r];
-          }
-        } else if (far) {
-          a1 = a2;
-        }
-        s[nb] = a1;
-      }
+      for (int kk = 0; kk < C::KSTEPS; ++kk)
+        a1 = hw::mfma32(operand_rowmajor<T, C::K_LD>(sK, nb * 32, 16 * kk, lane), qreg[kk], a1);
+      s[nb] = a1;
     }
+    hw::sched_prefetched_operands<(C::BN / 32) * C::KSTEPS, (C::KSTEPS >= 4 ? 4 : C::KSTEPS)>();
 
-    if (!PW) hw::sched_prefetched_operands<(C::BN / 32) * C::KSTEPS, (C::KSTEPS >= 4 ? 4 : C::KSTEPS)>();
-
-    // ---- masks (key tail, causal) only on tiles that need them ----
-    const bool need_mask = (n0 + C::BN > N) || (p.causal && (n0 + C::BN - 1 > pseq + mw));
+    // ---- masks (key tail, causal, the other regime's entries) only on tiles that need them ----
+    bool need_mask = (n0 + C::BN > N) || (p.causal && (n0 + C::BN - 1 > pseq + mw));
+    if (PW) need_mask = need_mask || (far_phase ? (mw + pseq - (n0 + C::BN - 1) < p.w) : (mw + 31 + pseq - n0 >= p.w));
     if (need_mask) {
 #pragma unroll
       for (int nb = 0; nb < C::BN / 32; ++nb)
@@ -178,6 +139,7 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (FwdCfg<T, D, PW>::WAVES_PER_SIMD)) f
         for (int r = 0; r < 16; ++r) {
           int n = n0 + nb * 32 + block_row(r, hh);
           bool keep = (n < N) && (!p.causal || (my_m + pseq >= n));
+          if (PW) keep = keep && ((my_m + pseq - n >= p.w) == far_phase);
           s[nb][r] = keep ? s[nb][r] : neg_inf();
         }
     }
@@ -226,11 +188,36 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (FwdCfg<T, D, PW>::WAVES_PER_SIMD)) f
           oacc[db] = hw::mfma32(operand_transposed<T, C::V_LD>(sV, nb * 32 + 16 * c, db * 32, lane), pb, oacc[db]);
       }
 
-    if (more) commit(n0 + C::BN, kStage ^ 1);
+    if (more) commit(kStage ^ 1);
     hw::block_sync();
   };
 
-  for (int it = 0; it < n_tiles; ++it) step(it, it & 1);
+  int stage = 0;
+#pragma unroll
+  for (int ph = 0; ph < (PW ? 2 : 1); ++ph) {
+    int t_begin = 0, t_end = n_tiles;
+    far_phase = PW && ph == 0;
+    if (PW) {
+      if (far_phase) {  // keys n <= m0 + BM - 1 + pseq - w are far from some row of the workgroup
+        const int far_hi = imin(hi, m0 + C::BM + pseq - p.w);
+        t_end = far_hi > 0 ? cdiv(far_hi, C::BN) : 0;
+      } else {          // keys n > m0 + pseq - w are near some row
+        t_begin = imax(0, m0 + pseq - p.w + 1) / C::BN;
+      }
+    }
+    if (t_begin >= t_end) continue;
+    k_src = far_phase ? k2b : kb;
+    k_stride = far_phase ? p.k2.st : p.k.st;
+    kr.init(tid, k_stride);
+    load_q(far_phase ? q2b : qb, far_phase ? p.q2.st : p.q.st);
+    fetch(t_begin * C::BN);
+    commit(stage);
+    hw::block_sync();
+    for (int it = t_begin; it < t_end; ++it) {
+      step(it, t_end, stage);
+      stage ^= 1;
+    }
+  }
 
   // ---- epilogue: O = acc / l, L = m * scale + ln(l); rows that saw no key give O = 0, L = -inf ----
   const float l_tot = l_i + hw::xor32(l_i);

@@ -11,7 +11,8 @@ import os
 import torch
 
 from . import _abi, _lib
-from .split_kv import num_splits_heuristic, split_kv_forward, SPLIT_BLOCK_M, SPLIT_BLOCK_N
+from .split_kv import (num_splits_heuristic, split_kv_forward, SPLIT_BLOCK_M, SPLIT_BLOCK_N,
+                       DECODE_MAX_ROWS)
 from .total import _total_attention
 
 __all__ = ["attention"]
@@ -56,7 +57,7 @@ class FlashAttention(torch.autograd.Function):
         with torch.cuda.device(q.device):
             num_cus = lib.fa_num_cus()
             splits = num_splits_heuristic(B, H, M, N, SPLIT_BLOCK_M, SPLIT_BLOCK_N, num_cus, 128)
-            if splits > 1:
+            if splits > 1 or (M <= DECODE_MAX_ROWS and N >= 1024):
                 o, L = split_kv_forward(lib, q, k, v, causal, sm_scale, splits)
             else:
                 o = torch.empty_like(q)

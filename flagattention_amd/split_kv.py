@@ -14,6 +14,10 @@ from . import _abi, _lib
 __all__ = ["attention"]
 
 SPLIT_BLOCK_M, SPLIT_BLOCK_N = 16, 128
+# Up to this many query positions the decode-shaped kernel is used even where the reference's rule
+# would not split: it multiplies 16-row tiles and reads K/V once per kv head, where the dense
+# forward kernel would fill 128-row tiles per query head with a handful of rows.
+DECODE_MAX_ROWS = 16
 
 
 def get_fwd_config(B, H, M, N, D, causal):
@@ -58,14 +62,14 @@ def _split_size(N, splits):
 def choose_num_splits(B, H, Hk, M, N, num_cus, reference_splits):
     """Number of pieces actually launched once the split path has been chosen.
 
-    The split kernel serves a whole GQA group (up to 32 query rows) from one workgroup, so it starts
-    ``B * Hk * ceil(G * M / 32)`` workgroups per split -- fewer than the per-query-head grid the
+    The split kernel serves a whole GQA group (up to 16 query rows) from one workgroup, so it starts
+    ``B * Hk * ceil(G * M / 16)`` workgroups per split -- fewer than the per-query-head grid the
     reference's rule assumes.  Splits are added until the launch has about four workgroups per
     compute unit, as long as every piece keeps at least 512 keys (four 32-key steps per wavefront).
     ``reference_splits`` (the count the reference's rule gives) is not used beyond having selected the
     split path.  The result of the operator does not depend on the count."""
     group = H // Hk
-    base = B * Hk * -(-(group * M) // 32)
+    base = B * Hk * -(-(group * M) // 16)
     n_units = -(-N // SPLIT_BLOCK_N)
     want = -(-4 * num_cus // base)
     cap = max(1, N // 512)
@@ -77,17 +81,19 @@ def choose_num_splits(B, H, Hk, M, N, num_cus, reference_splits):
     return splits
 
 
-def split_kv_forward(lib, q, k, v, causal, sm_scale, splits, combine=True):
-    """Runs the split kernel (+ merge).  Returns (o, L), or the fp16 partials when not merging."""
+def split_kv_forward(lib, q, k, v, causal, sm_scale, splits, single_direct=False):
+    """Runs the split kernel (+ merge) and returns (o, L).  ``splits`` is the count the reference's
+    rule gave; the number of pieces launched is chosen by ``choose_num_splits``.  With
+    ``single_direct`` a launch that ends up with one piece returns its fp16 partial output unmerged."""
     B, H, M, D = q.shape
     N = k.shape[2]
-    if splits > 1:
+    if splits != 1 or M <= DECODE_MAX_ROWS:
         splits = choose_num_splits(B, H, k.shape[1], M, N, lib.fa_num_cus(), splits)
     part_lse = torch.empty((B, H, splits, M), dtype=torch.float32, device=q.device)
     part_o = torch.empty((B, H, splits, M, D), dtype=torch.float16, device=q.device)
     _abi.fa_splitkv_fwd(lib, q, k, v, part_o, part_lse, causal, sm_scale, splits, _split_size(N, splits))
-    if not combine:
-        return part_o, part_lse
+    if single_direct and splits == 1:
+        return part_o.squeeze(2), part_lse.squeeze(2)
     L = torch.empty((B, H, M), dtype=torch.float32, device=q.device)
     o = torch.empty_like(q)
     if not _abi.is_kernel_ready(o):
@@ -114,8 +120,5 @@ def attention(q, k, v, causal=False, sm_scale=None):
     q, k, v = _abi.kernel_ready(q), _abi.kernel_ready(k), _abi.kernel_ready(v)
     with torch.cuda.device(q.device):
         splits = num_splits_heuristic(B, H, M, N, SPLIT_BLOCK_M, SPLIT_BLOCK_N, lib.fa_num_cus(), 128)
-        if splits == 1:
-            part_o, _ = split_kv_forward(lib, q, k, v, causal, sm_scale, 1, combine=False)
-            return part_o.squeeze(2)
-        o, _ = split_kv_forward(lib, q, k, v, causal, sm_scale, splits)
+        o, _ = split_kv_forward(lib, q, k, v, causal, sm_scale, splits, single_direct=True)
     return o

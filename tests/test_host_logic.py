@@ -6,7 +6,7 @@ import torch
 
 from flagattention_amd import _abi
 from flagattention_amd.paged import choose_launch, _next_pow2
-from flagattention_amd.split_kv import num_splits_heuristic, _split_size
+from flagattention_amd.split_kv import choose_num_splits, num_splits_heuristic, _split_size
 
 
 def brute_force_splits(B, H, M, N, bm, bn, cus, max_splits):
@@ -43,6 +43,18 @@ def test_known_split_counts():
 def test_split_size_covers_keys_in_128_key_units(N, S):
     size = _split_size(N, S)
     assert size % 128 == 0 and size * S >= N and size * (S - 1) < N + 128 * S
+
+
+def test_split_count_actually_launched():
+    # (B, H, Hk, M, N, compute units, reference count)
+    assert choose_num_splits(1, 32, 8, 1, 32768, 256, 8) == 64       # 8 workgroups per split -> cap N / 512
+    assert choose_num_splits(64, 32, 8, 1, 4096, 256, 1) == 2        # 512 workgroups per split
+    assert choose_num_splits(256, 32, 8, 1, 4096, 256, 1) == 1       # the batch alone fills the device
+    assert choose_num_splits(1, 8, 8, 4, 700, 256, 3) == 1           # pieces would be shorter than 512 keys
+    for args in [(1, 32, 8, 1, 32768, 256, 8), (2, 4, 2, 2, 4000, 256, 5), (1, 2, 1, 4, 8202, 256, 7)]:
+        s = choose_num_splits(*args)
+        n_units = -(-args[4] // 128)
+        assert 1 <= s <= 128 and (s == 1 or (-(-n_units // s)) * (s - 1) < n_units)   # no empty last piece
 
 
 def test_paged_launch_choice():

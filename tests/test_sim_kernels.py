@@ -140,6 +140,11 @@ PW_CASES = [
     (1, 1, 130, 260, 32, 100, False, torch.float16),
     (1, 1, 260, 130, 16, 190, True, torch.bfloat16),
     (1, 1, 150, 150, 128, -20, False, torch.float16),
+    (1, 1, 300, 300, 32, 70, True, torch.float16),      # threshold crosses several row and key blocks
+    (1, 1, 140, 200, 64, 0, True, torch.bfloat16),      # every visible pair is far
+    (1, 1, 140, 140, 16, 1000, True, torch.float16),    # every pair is near
+    (1, 1, 70, 330, 32, -1000, False, torch.bfloat16),  # non-causal, every pair far
+    (1, 1, 330, 70, 32, 129, False, torch.float16),     # M > N, threshold on a block edge
 ]
 
 
