@@ -117,6 +117,9 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (FwdCfg<T, D, PW>::WAVES_PER_SIMD)) f
     const T* sK = lds + kStage * C::STAGE;
     const T* sV = sK + C::K_TILE;
 
+    // A tile that the causal mask hides from all 32 rows of this wavefront (the last tiles of a
+    // workgroup, for its upper wavefronts) only takes part in the data movement.
+    if (!(p.causal && (mw + 31 + pseq < n0))) {
     // ---- S^T = K Q^T : BN/32 blocks of (32 keys x 32 queries) ----
     f32x16 s[C::BN / 32];
 #pragma unroll
@@ -188,6 +191,7 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (FwdCfg<T, D, PW>::WAVES_PER_SIMD)) f
           oacc[db] = hw::mfma32(operand_transposed<T, C::V_LD>(sV, nb * 32 + 16 * c, db * 32, lane), pb, oacc[db]);
       }
 
+    }
     if (more) commit(kStage ^ 1);
     hw::block_sync();
   };
