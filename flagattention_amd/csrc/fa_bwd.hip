@@ -73,7 +73,7 @@ struct KvCfg {
   static constexpr int BM = 64;   // queries per pipeline step
   static constexpr int DV = D < 32 ? 32 : D;
   static constexpr int KSTEPS = D / 16;
-  static constexpr int LD = DV + 40;  // rows 20 banks apart: 16-byte row reads conflict-free, transposing reads nearly so
+  static constexpr int LD = DV + (DV == 128 ? 24 : 40);  // 16-byte row reads and transposing reads both conflict-free
   static constexpr int TILE = BM * LD;
   // register budget: two wavefronts per SIMD (256 registers each) when the accumulators allow it
   static constexpr int WAVES_PER_SIMD = D <= 64 ? 2 : 1;
@@ -308,9 +308,9 @@ struct QCfg {
   static constexpr int BN = 64;   // keys per pipeline step
   static constexpr int DV = D < 32 ? 32 : D;
   static constexpr int KSTEPS = D / 16;
-  static constexpr int LD = DV + 40;  // rows 20 banks apart: 16-byte row reads conflict-free, transposing reads nearly so
+  static constexpr int LD = DV + (DV == 128 ? 24 : 40);  // 16-byte row reads and transposing reads both conflict-free
   static constexpr int TILE = BN * LD;
-  static constexpr int WAVES_PER_SIMD = (PW && D == 128) ? 1 : 2;  // the piecewise bookkeeping does not fit 256 registers at 128
+  static constexpr int WAVES_PER_SIMD = 2;
   static constexpr size_t STAGE_BYTES = 2 * TILE * sizeof(T);  // K, V
   static constexpr size_t LDS_BYTES = 2 * STAGE_BYTES;
 };
@@ -510,7 +510,7 @@ template <class T, int D>
 struct QdsCfg {
   static constexpr int BM = 128, BN = 64;
   static constexpr int DV = D < 32 ? 32 : D;
-  static constexpr int LD = DV + 40;
+  static constexpr int LD = DV + (DV == 128 ? 24 : 40);
   static constexpr int TILE = BN * LD;                 // K tile, elements
   static constexpr int VEC = 512 + 32 + 32;            // one chunk vector in the patch: 2 x (256 + 32 pad) elements
   static constexpr int PATCH = 2 * 2 * VEC;            // 2 chunks x 2 vectors per wavefront and stage
