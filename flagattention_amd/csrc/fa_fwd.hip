@@ -121,15 +121,15 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (FwdCfg<T, D, PW>::WAVES_PER_SIMD)) f
     // workgroup, for its upper wavefronts) only takes part in the data movement.
     if (!(p.causal && (mw + 31 + pseq < n0))) {
     // ---- S^T = K Q^T : BN/32 blocks of (32 keys x 32 queries) ----
+    // the two blocks advance together: consecutive matrix instructions never wait for each other
     f32x16 s[C::BN / 32];
 #pragma unroll
-    for (int nb = 0; nb < C::BN / 32; ++nb) {
-      f32x16 a1 = zero16;
+    for (int nb = 0; nb < C::BN / 32; ++nb) s[nb] = zero16;
 #pragma unroll
-      for (int kk = 0; kk < C::KSTEPS; ++kk)
-        a1 = hw::mfma32(operand_rowmajor<T, C::K_LD>(sK, nb * 32, 16 * kk, lane), qreg[kk], a1);
-      s[nb] = a1;
-    }
+    for (int kk = 0; kk < C::KSTEPS; ++kk)
+#pragma unroll
+      for (int nb = 0; nb < C::BN / 32; ++nb)
+        s[nb] = hw::mfma32(operand_rowmajor<T, C::K_LD>(sK, nb * 32, 16 * kk, lane), qreg[kk], s[nb]);
     hw::sched_prefetched_operands<(C::BN / 32) * C::KSTEPS, (C::KSTEPS >= 4 ? 4 : C::KSTEPS)>();
 
     // ---- masks (key tail, causal, the other regime's entries) only on tiles that need them ----
