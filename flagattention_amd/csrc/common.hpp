@@ -26,47 +26,14 @@ FA_DEVICE float neg_inf() { return -__builtin_inff(); }
 // ---------------------------------------------------------------------------------------------
 // global -> registers -> LDS movement of a ROWS x COLS tile (16 bytes per thread per step)
 // ---------------------------------------------------------------------------------------------
-template <int ROWS, int COLS>
-struct TileRegs {
-  static constexpr int kChunks = ROWS * COLS / 8;
-  static constexpr int kPerThread = (kChunks + kThreads - 1) / kThreads;
-  u32x4 r[kPerThread];
-};
-
-// Rows at or beyond `row_limit` are filled with zeros (a masked probability times a stray NaN
-// would otherwise poison the accumulators).
-template <class T, int ROWS, int COLS>
-FA_DEVICE void tile_fetch(TileRegs<ROWS, COLS>& t, const T* base, int64_t row_stride, int row0,
-                          int row_limit, int tid) {
-  constexpr int kCPR = COLS / 8;  // 16-byte chunks per row
-#pragma unroll
-  for (int i = 0; i < TileRegs<ROWS, COLS>::kPerThread; ++i) {
-    int c = tid + i * kThreads;
-    u32x4 v = {0u, 0u, 0u, 0u};
-    if (c < TileRegs<ROWS, COLS>::kChunks) {
-      int r = c / kCPR, col = (c % kCPR) * 8;
-      if (row0 + r < row_limit) v = *(const u32x4*)(base + (int64_t)(row0 + r) * row_stride + col);
-    }
-    t.r[i] = v;
-  }
-}
-
-template <class T, int ROWS, int COLS, int LD>
-FA_DEVICE void tile_commit(const TileRegs<ROWS, COLS>& t, T* lds_tile, int tid) {
-  constexpr int kCPR = COLS / 8;
-#pragma unroll
-  for (int i = 0; i < TileRegs<ROWS, COLS>::kPerThread; ++i) {
-    int c = tid + i * kThreads;
-    if (c < TileRegs<ROWS, COLS>::kChunks) {
-      int r = c / kCPR, col = (c % kCPR) * 8;
-      *(u32x4*)(lds_tile + r * LD + col) = t.r[i];
-    }
-  }
-}
-
 // Loop-invariant plan of one thread's share of a ROWS x COLS tile: byte offsets inside the global
 // tile are computed once, so that a steady-state fetch is one load per chunk from a uniform tile
 // base plus a 32-bit lane offset, and the LDS destination is a fixed offset from the tile start.
+//
+// fetch() is branch-free on purpose.  With a branch per load (or per tile kind) the compiler puts
+// loads in separate basic blocks and waits for ALL outstanding loads at their boundaries -- a full
+// memory latency per tile.  Rows that do not exist are therefore read from the last row that does
+// (always valid memory) and replaced by zeros when the tile is committed to LDS.
 template <class T, int ROWS, int COLS>
 struct TileMover {
   static constexpr int CPR = COLS / 8;          // 16-byte chunks per row
@@ -75,39 +42,37 @@ struct TileMover {
   static constexpr bool kExact = (PASSES * RPP == ROWS);
   u32x4 r[PASSES];
   uint32_t goff[PASSES];
+  uint32_t stride_bytes, col_bytes;
   int row0, col0;
+  int valid;  // rows of the fetched tile that exist
 
   FA_DEVICE void init(int tid, int64_t row_stride) {
     row0 = tid / CPR;
     col0 = (tid % CPR) * 8;
+    stride_bytes = (uint32_t)(row_stride * (int64_t)sizeof(T));
+    col_bytes = (uint32_t)(col0 * (int)sizeof(T));
+    valid = ROWS;
 #pragma unroll
-    for (int i = 0; i < PASSES; ++i)
-      goff[i] = (uint32_t)(((int64_t)(row0 + i * RPP) * row_stride + col0) * (int64_t)sizeof(T));
+    for (int i = 0; i < PASSES; ++i) goff[i] = (uint32_t)(row0 + i * RPP) * stride_bytes + col_bytes;
   }
-  // every row of the tile exists
-  FA_DEVICE void fetch_full(const T* tile_base) {
-#pragma unroll
-    for (int i = 0; i < PASSES; ++i) {
-      u32x4 v = {0u, 0u, 0u, 0u};
-      if (kExact || row0 + i * RPP < ROWS) v = *(const u32x4*)((const char*)tile_base + goff[i]);
-      r[i] = v;
-    }
-  }
-  // only the first rows_valid rows exist; the rest is filled with zeros
-  FA_DEVICE void fetch_rows(const T* tile_base, int rows_valid) {
-#pragma unroll
-    for (int i = 0; i < PASSES; ++i) {
-      u32x4 v = {0u, 0u, 0u, 0u};
-      const int row = row0 + i * RPP;
-      if ((kExact || row < ROWS) && row < rows_valid) v = *(const u32x4*)((const char*)tile_base + goff[i]);
-      r[i] = v;
-    }
-  }
+  // rows_valid >= 1 rows of the tile exist
   FA_DEVICE void fetch(const T* tile_base, int rows_valid) {
-    if (rows_valid >= ROWS) fetch_full(tile_base); else fetch_rows(tile_base, rows_valid);
+    valid = rows_valid < ROWS ? rows_valid : ROWS;
+    const uint32_t last = (uint32_t)(valid - 1) * stride_bytes + col_bytes;
+#pragma unroll
+    for (int i = 0; i < PASSES; ++i) {
+      const uint32_t off = (row0 + i * RPP < valid) ? goff[i] : last;
+      r[i] = *(const u32x4*)((const char*)tile_base + off);
+    }
   }
   template <int LD>
-  FA_DEVICE void commit(T* lds_tile) const {
+  FA_DEVICE void commit(T* lds_tile) {
+    if (valid < ROWS) {  // tail tile only (uniform): rows past the end become zeros
+      hw::keep_branch();
+#pragma unroll
+      for (int i = 0; i < PASSES; ++i)
+        if (row0 + i * RPP >= valid) r[i] = u32x4{0u, 0u, 0u, 0u};
+    }
 #pragma unroll
     for (int i = 0; i < PASSES; ++i)
       if (kExact || row0 + i * RPP < ROWS) *(u32x4*)(lds_tile + (row0 + i * RPP) * LD + col0) = r[i];

@@ -151,16 +151,17 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (KvCfg<T, D, PW>::WAVES_PER_SIMD)) fa
   TileMover<T, C::BM, D> qr, gr;
   gr.init(tid, p.dout.st);
   float l_reg = 0.f, d_reg = 0.f;
+  int l_row = 0;
   auto fetch = [&](int m0) {
     const int rows = M - m0;
     qr.fetch(q_src + (int64_t)m0 * q_stride, rows);
     gr.fetch(gb + (int64_t)m0 * p.dout.st, rows);
-    if (tid < C::BM) {
-      int m = m0 + tid;
-      // rows past M get L = +inf, hence P = 0
-      l_reg = m < M ? lse[m] * kLog2e : __builtin_inff();
-      d_reg = m < M ? dlt[m] : 0.f;
-    }
+    // L and delta of row m0 + tid (threads 0..63), read branch-free from a clamped row and fixed up
+    // at commit: nothing may consume a load here, or the wait would cover the tile loads as well
+    l_row = m0 + (tid & (C::BM - 1));
+    const int mc = imin(l_row, M - 1);
+    l_reg = lse[mc];
+    d_reg = dlt[mc];
   };
   auto commit = [&](int stage) {
     unsigned char* base = smem + stage * C::STAGE_BYTES;
@@ -168,7 +169,11 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (KvCfg<T, D, PW>::WAVES_PER_SIMD)) fa
     qr.template commit<C::LD>(s);
     gr.template commit<C::LD>(s + C::TILE);
     float* f = (float*)(base + 2 * C::TILE * sizeof(T));
-    if (tid < C::BM) { f[tid] = l_reg; f[C::BM + tid] = d_reg; }
+    // rows past M get L = +inf, hence P = 0
+    if (tid < C::BM) {
+      f[tid] = l_row < M ? l_reg * kLog2e : __builtin_inff();
+      f[C::BM + tid] = l_row < M ? d_reg : 0.f;
+    }
   };
 
   const float c2 = p.sm_scale * kLog2e;
@@ -210,6 +215,7 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (KvCfg<T, D, PW>::WAVES_PER_SIMD)) fa
       commit(stage);
       hw::block_sync();
     }
+    hw::wait_global_loads();  // K and V rows
 
     for (int it = t_begin; it < t_end; ++it) {
       const int m0 = it * C::BM;
@@ -428,6 +434,7 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (QCfg<T, D, PW>::WAVES_PER_SIMD)) fa_
       commit(stage);
       hw::block_sync();
     }
+    hw::wait_global_loads();  // Q and dO rows
 
     for (int it = t_begin; it < t_end; ++it) {
       const int n0 = it * C::BN;

@@ -217,6 +217,7 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (FwdCfg<T, D, PW>::WAVES_PER_SIMD)) f
     fetch(t_begin * C::BN);
     commit(stage);
     hw::block_sync();
+    hw::wait_global_loads();  // Q rows
     for (int it = t_begin; it < t_end; ++it) {
       step(it, t_end, stage);
       stage ^= 1;

@@ -50,23 +50,26 @@ FA_KERNEL void FA_LAUNCH_BOUNDS(kThreads) fa_total_kernel(TotalParams p) {
   if (p.causal) m_lo = (imax(0, n0 - pseq) / C::BM) * C::BM;
   const int n_tiles = m_lo < M ? cdiv(M - m_lo, C::BM) : 0;
 
-  TileRegs<C::BM, D> qr;
+  TileMover<T, C::BM, D> qr;
+  qr.init(tid, p.q.st);
   float l_reg = 0.f;
+  int l_row = 0;
   auto fetch = [&](int m0) {
-    tile_fetch<T, C::BM, D>(qr, qb, p.q.st, m0, M, tid);
-    if (tid < C::BM) {
-      int m = m0 + tid;
-      l_reg = m < M ? lse[m] * kLog2e : __builtin_inff();  // rows past M: P = 0
-    }
+    qr.fetch(qb + (int64_t)m0 * p.q.st, M - m0);
+    // branch-free, and nothing consumes the load here (the wait would cover the tile loads too)
+    l_row = m0 + (tid & (C::BM - 1));
+    l_reg = lse[imin(l_row, M - 1)];
   };
   auto commit = [&](int stage) {
     unsigned char* base = smem + stage * C::STAGE_BYTES;
-    tile_commit<T, C::BM, D, C::LD>(qr, (T*)base, tid);
-    if (tid < C::BM) ((float*)(base + C::TILE * sizeof(T)))[tid] = l_reg;
+    qr.template commit<C::LD>((T*)base);
+    // rows past M: P = 0
+    if (tid < C::BM) ((float*)(base + C::TILE * sizeof(T)))[tid] = l_row < M ? l_reg * kLog2e : __builtin_inff();
   };
 
   if (n_tiles > 0) { fetch(m_lo); commit(0); }
   hw::block_sync();
+  hw::wait_global_loads();  // K rows
 
   const float c2 = p.sm_scale * kLog2e;
   float colsum = 0.f;

@@ -95,6 +95,11 @@ FA_DEVICE int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
 FA_DEVICE void store_streaming(void* p, u32x4 v) { __builtin_nontemporal_store(v, (u32x4*)p); }
 FA_DEVICE u32x4 load_streaming(const void* p) { return __builtin_nontemporal_load((const u32x4*)p); }
 
+// Waits until every global load issued so far has delivered its registers.  Placed between the
+// loads of loop-invariant operands and a loop that also prefetches: otherwise the compiler puts the
+// wait at the operands' first use INSIDE the loop, where it also covers the prefetch just issued.
+FA_DEVICE void wait_global_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // vmcnt(0), others unconstrained
+
 // Marks a branch body as not speculatable, so that a wavefront-uniform `if` stays a branch instead
 // of being turned into unconditional arithmetic on selected operands.
 FA_DEVICE void keep_branch() { asm volatile("" ::: "memory"); }

@@ -198,6 +198,7 @@ inline int block_z() { return hwsim::bz; }
 inline int grid_x() { return hwsim::gx; }
 inline void store_streaming(void* p, u32x4 v) { *(u32x4*)p = v; }
 inline u32x4 load_streaming(const void* p) { return *(const u32x4*)p; }
+inline void wait_global_loads() {}
 inline int uniform(int x) { return x; }
 inline int grid_z() { return hwsim::gz; }
 inline void block_sync() { hwsim::yield(hwsim::OP_BARRIER); }
