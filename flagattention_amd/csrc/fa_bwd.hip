@@ -411,7 +411,7 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (QCfg<T, D, PW>::WAVES_PER_SIMD)) fa_
   };
 
   int stage = 0;
-#pragma unroll
+#pragma unroll 1
   for (int ph = 0; ph < (PW ? 2 : 1); ++ph) {
     far_phase = PW && ph == 0;
     int t_begin = 0, t_end = n_tiles;

@@ -197,7 +197,7 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (FwdCfg<T, D, PW>::WAVES_PER_SIMD)) f
   };
 
   int stage = 0;
-#pragma unroll
+#pragma unroll 1
   for (int ph = 0; ph < (PW ? 2 : 1); ++ph) {
     int t_begin = 0, t_end = n_tiles;
     far_phase = PW && ph == 0;
