@@ -203,6 +203,24 @@ def paged_bench(torch, iters=50):
                          "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": PAGED_TRAFFIC_BYTES}}
 
 
+def splitkv_bench(torch, iters=50):
+    """Dense split-KV decode through flash_attention: q (4, 32, 1, 128), k/v (4, 8, 32768, 128) fp16."""
+    import flagattention_amd as flag_attn
+    dev = "cuda:0"
+    g = torch.Generator(device=dev).manual_seed(10086)
+    B, H, Hk, N, D = 4, 32, 8, 32768, 128
+    q = torch.randn(B, H, 1, D, device=dev, dtype=torch.float16, generator=g)
+    k = torch.randn(B, Hk, N, D, device=dev, dtype=torch.float16, generator=g)
+    v = torch.randn(B, Hk, N, D, device=dev, dtype=torch.float16, generator=g)
+    ms = timed_launches(lambda: flag_attn.flash_attention(q, k, v, causal=False), iters, torch)
+    algo = 2 * k.numel() * 2 + 2 * q.numel() * 2
+    gbs = algo / (ms * 1e-3) / 1e9
+    return {"workload": "flash_attention decode fp16 q=(4,32,1,128) k/v=(4,8,32768,128) (split-KV path)",
+            "ms": round(ms, 4), "algorithmic_bytes": algo, "value": round(gbs, 1), "unit": "GB/s",
+            "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                         "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None}}
+
+
 def profile_kernel(args, torch):
     """A handful of launches of one kernel at the benchmark's shapes, nothing else on the device."""
     from flagattention_amd import _abi, _lib
@@ -279,6 +297,7 @@ def main():
     }
     if not args.no_paged:
         out["paged_decode"] = paged_bench(torch)
+        out["splitkv_decode"] = splitkv_bench(torch)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args, torch)
     print(json.dumps(out))
