@@ -48,7 +48,8 @@ def test_split_size_covers_keys_in_128_key_units(N, S):
 def test_split_count_actually_launched():
     # (B, H, Hk, M, N, compute units, reference count)
     assert choose_num_splits(1, 32, 8, 1, 32768, 256, 8) == 64       # 8 workgroups per split -> cap N / 512
-    assert choose_num_splits(64, 32, 8, 1, 4096, 256, 1) == 2        # 512 workgroups per split
+    assert choose_num_splits(64, 32, 8, 1, 4096, 256, 1) == 1        # 512 workgroups: one resident wave already
+    assert choose_num_splits(4, 32, 8, 1, 32768, 256, 2) == 16       # 32 workgroups per split -> 512
     assert choose_num_splits(256, 32, 8, 1, 4096, 256, 1) == 1       # the batch alone fills the device
     assert choose_num_splits(1, 8, 8, 4, 700, 256, 3) == 1           # pieces would be shorter than 512 keys
     for args in [(1, 32, 8, 1, 32768, 256, 8), (2, 4, 2, 2, 4000, 256, 5), (1, 2, 1, 4, 8202, 256, 7)]:
