@@ -88,12 +88,19 @@ def fa_bwd_delta(lib, o, do, delta):
           "fa_bwd_delta")
 
 
+def _heads_per_slice(q, dk):
+    """dk / dv hold one slice per this many query heads (summed by the kernel)."""
+    H, slices = q.shape[1], dk.shape[1]
+    assert H % slices == 0
+    return H // slices
+
+
 def fa_bwd_dkdv(lib, q, k, v, do, lse, delta, dk, dv, causal, sm_scale):
     B, H, M, D = q.shape
     Hk, N = k.shape[1], k.shape[2]
     check(lib.fa_bwd_dkdv(dtype_code(q), view4(q), view4(k), view4(v), view4(do), ptr(lse), ptr(delta),
-                          view4(dk), view4(dv), B, H, Hk, M, N, D, int(causal), float(sm_scale),
-                          stream_of(q)), "fa_bwd_dkdv")
+                          view4(dk), view4(dv), _heads_per_slice(q, dk), B, H, Hk, M, N, D, int(causal),
+                          float(sm_scale), stream_of(q)), "fa_bwd_dkdv")
 
 
 def fa_bwd_dq(lib, q, k, v, do, lse, delta, dq, causal, sm_scale):
@@ -108,8 +115,9 @@ def fa_bwd_dkdv_ds(lib, q, k, v, do, lse, delta, dk, dv, ds, causal, sm_scale):
     B, H, M, D = q.shape
     Hk, N = k.shape[1], k.shape[2]
     check(lib.fa_bwd_dkdv_ds(dtype_code(q), view4(q), view4(k), view4(v), view4(do), ptr(lse), ptr(delta),
-                             view4(dk), view4(dv), ptr(ds), ds.numel() * ds.element_size(), B, H, Hk, M,
-                             N, D, int(causal), float(sm_scale), stream_of(q)), "fa_bwd_dkdv_ds")
+                             view4(dk), view4(dv), _heads_per_slice(q, dk), ptr(ds),
+                             ds.numel() * ds.element_size(), B, H, Hk, M, N, D, int(causal),
+                             float(sm_scale), stream_of(q)), "fa_bwd_dkdv_ds")
 
 
 def fa_bwd_dq_from_ds(lib, k, ds, dq, causal, sm_scale):

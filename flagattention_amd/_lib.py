@@ -25,10 +25,10 @@ SIGNATURES = {
     "fa_num_cus": [],
     "fa_fwd": [_i, _v, _v, _v, _v, _p, _i, _i, _i, _i, _i, _i, _i, _f, _p],
     "fa_bwd_delta": [_i, _v, _v, _p, _i, _i, _i, _i, _p],
-    "fa_bwd_dkdv": [_i, _v, _v, _v, _v, _p, _p, _v, _v, _i, _i, _i, _i, _i, _i, _i, _f, _p],
+    "fa_bwd_dkdv": [_i, _v, _v, _v, _v, _p, _p, _v, _v, _i, _i, _i, _i, _i, _i, _i, _i, _f, _p],
     "fa_bwd_dq": [_i, _v, _v, _v, _v, _p, _p, _v, _i, _i, _i, _i, _i, _i, _i, _f, _p],
     "fa_bwd_ds_workspace_mib": [_i, _i, _i, _i],
-    "fa_bwd_dkdv_ds": [_i, _v, _v, _v, _v, _p, _p, _v, _v, _p, _i64, _i, _i, _i, _i, _i, _i, _i, _f, _p],
+    "fa_bwd_dkdv_ds": [_i, _v, _v, _v, _v, _p, _p, _v, _v, _i, _p, _i64, _i, _i, _i, _i, _i, _i, _i, _f, _p],
     "fa_bwd_dq_from_ds": [_i, _v, _p, _i64, _v, _i, _i, _i, _i, _i, _i, _i, _f, _p],
     "fa_total_attn": [_i, _v, _v, _p, _p, _i, _i, _i, _i, _i, _i, _i, _f, _p],
     "fa_splitkv_fwd": [_i, _v, _v, _v, _p, _p, _i, _i, _i, _i, _i, _i, _i, _f, _i, _i, _p],

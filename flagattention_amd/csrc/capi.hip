@@ -99,13 +99,14 @@ static int fill_bwd(fa::BwdParams& p, int dtype, const fa_view4* q, const fa_vie
 
 int fa_bwd_dkdv(int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v,
                 const fa_view4* dout, const float* lse, const float* delta, const fa_view4* dk,
-                const fa_view4* dv, int B, int H, int Hk, int M, int N, int D, int causal,
-                float sm_scale, void* stream) {
+                const fa_view4* dv, int heads_per_slice, int B, int H, int Hk, int M, int N, int D,
+                int causal, float sm_scale, void* stream) {
   fa::BwdParams p = {};
   int rc = fill_bwd(p, dtype, q, k, v, dout, lse, delta, B, H, Hk, M, N, D, causal, sm_scale);
   if (rc) return rc;
   if (!view_ok(dk) || !view_ok(dv)) return FA_ERR_BAD_ARGUMENT;
   p.dk = to_view(dk); p.dv = to_view(dv);
+  p.chunk = heads_per_slice;
   return fa::run_bwd_dkdv(p, false, (hipStream_t)stream);
 }
 
@@ -128,8 +129,8 @@ int fa_bwd_ds_workspace_mib(int B, int H, int M, int N) {
 
 int fa_bwd_dkdv_ds(int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v,
                    const fa_view4* dout, const float* lse, const float* delta, const fa_view4* dk,
-                   const fa_view4* dv, void* ds_workspace, int64_t ds_workspace_bytes, int B, int H,
-                   int Hk, int M, int N, int D, int causal, float sm_scale, void* stream) {
+                   const fa_view4* dv, int heads_per_slice, void* ds_workspace, int64_t ds_workspace_bytes,
+                   int B, int H, int Hk, int M, int N, int D, int causal, float sm_scale, void* stream) {
   fa::BwdParams p = {};
   int rc = fill_bwd(p, dtype, q, k, v, dout, lse, delta, B, H, Hk, M, N, D, causal, sm_scale);
   if (rc) return rc;
@@ -138,6 +139,7 @@ int fa_bwd_dkdv_ds(int dtype, const fa_view4* q, const fa_view4* k, const fa_vie
       ds_workspace_bytes < fa::bwd_ds_workspace_bytes(B, H, M, N))
     return FA_ERR_BAD_ARGUMENT;
   p.dk = to_view(dk); p.dv = to_view(dv);
+  p.chunk = heads_per_slice;
   p.ds = ds_workspace;
   return fa::run_bwd_dkdv_ds(p, (hipStream_t)stream);
 }

@@ -99,16 +99,22 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (KvCfg<T, D, PW>::WAVES_PER_SIMD)) fa
 
   const int tid = hw::thread_id(), lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, hh = lane >> 5;
-  const TileId wg = tile_of_workgroup(p.H, p.B);  // key blocks in ascending order: most queries first
-  const int head = wg.head, batch = wg.batch;
-  const int hk = head / p.group;
+  // One workgroup per (key block, chunk of query heads that share a kv head): it walks the heads of
+  // the chunk one after the other and accumulates their dK / dV in the same registers, so the sum
+  // over the chunk costs nothing.  chunk = group gives dK/dV per kv head; smaller chunks (more
+  // workgroups, for launches that would not fill the device) leave group / chunk slices to add.
+  const int chunk = p.chunk > 0 ? p.chunk : p.group;
+  const TileId wg = tile_of_workgroup(p.H / chunk, p.B);  // key blocks in ascending order: most queries first
+  const int slice = wg.head, batch = wg.batch;             // output slice = chunk index
+  const int hk = slice * chunk / p.group;
   const int M = p.M, N = p.N, pseq = N - M;
   const int n0 = wg.rank * C::BN, nw = n0 + wave * 32, my_n = nw + l32;
 
-  const T* gb = (const T*)p.dout.ptr + batch * p.dout.sb + head * p.dout.sh;
+  int head = slice * chunk;  // query head being processed
+  const T* gb = nullptr;
   const T* vb = (const T*)p.v.ptr + batch * p.v.sb + hk * p.v.sh;
-  const float* lse = p.lse + ((int64_t)batch * p.H + head) * M;
-  const float* dlt = p.delta + ((int64_t)batch * p.H + head) * M;
+  const float* lse = nullptr;
+  const float* dlt = nullptr;
 
   // K (of the current regime) and V rows of this lane as B operands (k = 16 kk + 8 hh + 0..7)
   V8 kreg[C::KSTEPS], vreg[C::KSTEPS];
@@ -140,10 +146,6 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (KvCfg<T, D, PW>::WAVES_PER_SIMD)) fa
 
   // dS chunks of this wavefront's key block: one row of the (key block, query block) chunk grid
   T* ds_row = nullptr;
-  if (DS) {
-    const int64_t nqb = 4 * (int64_t)cdiv(M, 128), nkb = 4 * (int64_t)cdiv(N, 128);
-    ds_row = (T*)p.ds + ((((int64_t)batch * p.H + head) * nkb + (n0 / 32 + wave)) * nqb) * 1024 + lane * 8;
-  }
 
   bool far_phase = false;
   const T* q_src = nullptr;
@@ -180,7 +182,7 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (KvCfg<T, D, PW>::WAVES_PER_SIMD)) fa
 
   // result block (keys x D): D along lanes, keys along registers
   auto store_keys = [&](const f32x16* acc, const View4& dst, float scale) {
-    T* base = (T*)dst.ptr + batch * dst.sb + head * dst.sh;
+    T* base = (T*)dst.ptr + batch * dst.sb + slice * dst.sh;
 #pragma unroll
     for (int db = 0; db < C::DV / 32; ++db) {
       const int d = db * 32 + l32;
@@ -195,6 +197,16 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (KvCfg<T, D, PW>::WAVES_PER_SIMD)) fa
   };
 
   int stage = 0;
+#pragma unroll 1
+  for (int gi = 0; gi < chunk; ++gi) {
+  head = slice * chunk + gi;
+  gb = (const T*)p.dout.ptr + batch * p.dout.sb + head * p.dout.sh;
+  lse = p.lse + ((int64_t)batch * p.H + head) * M;
+  dlt = p.delta + ((int64_t)batch * p.H + head) * M;
+  if (DS) {
+    const int64_t nqb = 4 * (int64_t)cdiv(M, 128), nkb = 4 * (int64_t)cdiv(N, 128);
+    ds_row = (T*)p.ds + ((((int64_t)batch * p.H + head) * nkb + (n0 / 32 + wave)) * nqb) * 1024 + lane * 8;
+  }
 #pragma unroll
   for (int ph = 0; ph < (PW ? 2 : 1); ++ph) {
     far_phase = PW && ph == 1;
@@ -295,15 +307,18 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (KvCfg<T, D, PW>::WAVES_PER_SIMD)) fa
       stage ^= 1;
     }
 
-    // this regime's dK is complete
-    store_keys(dk, (PW && far_phase) ? p.dk2 : p.dk, p.sm_scale);
-    if (PW && !far_phase) {
+    if (PW) {  // this regime's dK is complete (piecewise has no grouped heads)
+      store_keys(dk, far_phase ? p.dk2 : p.dk, p.sm_scale);
+      if (!far_phase) {
 #pragma unroll
-      for (int i = 0; i < C::DV / 32; ++i)
+        for (int i = 0; i < C::DV / 32; ++i)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) dk[i][r] = 0.f;
+          for (int r = 0; r < 16; ++r) dk[i][r] = 0.f;
+      }
     }
   }
+  }
+  if (!PW) store_keys(dk, p.dk, p.sm_scale);
   store_keys(dv, p.dv, 1.f);
 }
 
@@ -643,7 +658,7 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, 2) fa_bwd_dq_from_ds_kernel(BwdParams
 // ------------------------------------------------------------------------------ launchers ----
 template <class T, bool PW>
 static int launch_dkdv(const BwdParams& p, hipStream_t stream) {
-  dim3 grid(((p.N + 127) / 128) * p.H * p.B, 1, 1);
+  dim3 grid(((p.N + 127) / 128) * (p.H / (p.chunk > 0 ? p.chunk : p.group)) * p.B, 1, 1);
   switch (p.D) {
     case 16: return launch(fa_bwd_dkdv_kernel<T, 16, PW>, grid, KvCfg<T, 16, PW>::LDS_BYTES, stream, p);
     case 32: return launch(fa_bwd_dkdv_kernel<T, 32, PW>, grid, KvCfg<T, 32, PW>::LDS_BYTES, stream, p);
@@ -667,6 +682,7 @@ static int launch_dq(const BwdParams& p, hipStream_t stream) {
 
 int run_bwd_dkdv(const BwdParams& p, bool piecewise, hipStream_t stream) {
   if (p.B <= 0 || p.H <= 0 || p.M <= 0 || p.N <= 0 || p.group <= 0) return kBadArgument;
+  if (p.chunk < 0 || (p.chunk > 0 && p.group % p.chunk)) return kBadArgument;
   if (p.dtype == kDtypeF16)
     return piecewise ? launch_dkdv<hw::half_t, true>(p, stream) : launch_dkdv<hw::half_t, false>(p, stream);
   if (p.dtype == kDtypeBF16)
@@ -685,7 +701,7 @@ int run_bwd_dq(const BwdParams& p, bool piecewise, hipStream_t stream) {
 
 template <class T>
 static int launch_dkdv_ds(const BwdParams& p, hipStream_t stream) {
-  dim3 grid(((p.N + 127) / 128) * p.H * p.B, 1, 1);
+  dim3 grid(((p.N + 127) / 128) * (p.H / (p.chunk > 0 ? p.chunk : p.group)) * p.B, 1, 1);
   switch (p.D) {
     case 16: return launch(fa_bwd_dkdv_kernel<T, 16, false, true>, grid, KvCfg<T, 16, false>::LDS_BYTES, stream, p);
     case 32: return launch(fa_bwd_dkdv_kernel<T, 32, false, true>, grid, KvCfg<T, 32, false>::LDS_BYTES, stream, p);
@@ -713,6 +729,7 @@ int64_t bwd_ds_workspace_bytes(int B, int H, int M, int N) {
 
 int run_bwd_dkdv_ds(const BwdParams& p, hipStream_t stream) {
   if (p.B <= 0 || p.H <= 0 || p.M <= 0 || p.N <= 0 || p.group <= 0 || !p.ds) return kBadArgument;
+  if (p.chunk < 0 || (p.chunk > 0 && p.group % p.chunk)) return kBadArgument;
   if (p.dtype == kDtypeF16) return launch_dkdv_ds<hw::half_t>(p, stream);
   if (p.dtype == kDtypeBF16) return launch_dkdv_ds<hw::bf16_t>(p, stream);
   return kUnsupported;

@@ -25,12 +25,13 @@ struct FwdParams {
 
 struct BwdParams {
   View4 q, k, v, q2, k2, o, dout;
-  View4 dq, dk, dv, dq2, dk2;  // written; dk/dv have one slice per *query* head
+  View4 dq, dk, dv, dq2, dk2;  // written; dk/dv have one slice per `chunk` query heads
   const float* lse;            // (B, H, M)
   float* delta;                // (B, H, M) rowsum(O * dO): written by the preprocess, read by the rest
   void* ds;                    // optional dS workspace: written by the dK/dV kernel, read by dQ-from-dS
   int B, H, M, N, D;
   int group;
+  int chunk;  // query heads whose dK/dV one workgroup accumulates (divides group; 0 = group)
   int causal;
   int w;
   float sm_scale;

@@ -56,16 +56,20 @@ int fa_fwd(int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v, c
  * The reference's three launches in FlashAttention.backward, src/flag_attn/flash.py:191-249:
  *
  * fa_bwd_delta  <- `_bwd_preprocess` (flash.py:522-568): delta[b,h,m] = sum_d o * dout, fp32.
- * fa_bwd_dkdv   <- `_bwd_kv_kernel`  (flash.py:571-745): dk, dv of shape (B, H, N, D), one slice per
- *                  QUERY head; the caller sums groups of H / Hk slices (flash.py:250-251).
+ * fa_bwd_dkdv   <- `_bwd_kv_kernel`  (flash.py:571-745) and, in part or in full, the group reduction
+ *                  that follows it (flash.py:205-206, 250-251): dk, dv of shape
+ *                  (B, H / heads_per_slice, N, D); slice s is the sum over query heads
+ *                  s * heads_per_slice ... + heads_per_slice - 1 (fp32 accumulation inside the kernel).
+ *                  heads_per_slice must divide H / Hk; 0 means H / Hk (one slice per kv head);
+ *                  1 reproduces the reference's one slice per query head.
  * fa_bwd_dq     <- `_bwd_q_kernel`   (flash.py:748-909): dq (B, H, M, D), every element written.
  * No atomics; each workgroup owns its output tile. */
 int fa_bwd_delta(int dtype, const fa_view4* o, const fa_view4* dout, float* delta, int B, int H,
                  int M, int D, void* stream);
 int fa_bwd_dkdv(int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v,
                 const fa_view4* dout, const float* lse, const float* delta, const fa_view4* dk,
-                const fa_view4* dv, int B, int H, int Hk, int M, int N, int D, int causal,
-                float sm_scale, void* stream);
+                const fa_view4* dv, int heads_per_slice, int B, int H, int Hk, int M, int N, int D,
+                int causal, float sm_scale, void* stream);
 int fa_bwd_dq(int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v,
               const fa_view4* dout, const float* lse, const float* delta, const fa_view4* dq, int B,
               int H, int Hk, int M, int N, int D, int causal, float sm_scale, void* stream);
@@ -81,8 +85,8 @@ int fa_bwd_dq(int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v
 int fa_bwd_ds_workspace_mib(int B, int H, int M, int N);
 int fa_bwd_dkdv_ds(int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v,
                    const fa_view4* dout, const float* lse, const float* delta, const fa_view4* dk,
-                   const fa_view4* dv, void* ds_workspace, int64_t ds_workspace_bytes, int B, int H,
-                   int Hk, int M, int N, int D, int causal, float sm_scale, void* stream);
+                   const fa_view4* dv, int heads_per_slice, void* ds_workspace, int64_t ds_workspace_bytes,
+                   int B, int H, int Hk, int M, int N, int D, int causal, float sm_scale, void* stream);
 int fa_bwd_dq_from_ds(int dtype, const fa_view4* k, const void* ds_workspace, int64_t ds_workspace_bytes,
                       const fa_view4* dq, int B, int H, int Hk, int M, int N, int D, int causal,
                       float sm_scale, void* stream);

@@ -58,6 +58,18 @@ def test_split_count_actually_launched():
         assert 1 <= s <= 128 and (s == 1 or (-(-n_units // s)) * (s - 1) < n_units)   # no empty last piece
 
 
+def test_dkdv_heads_per_slice():
+    from flagattention_amd.flash import dkdv_heads_per_slice
+    # (B, H, group, N, compute units)
+    assert dkdv_heads_per_slice(1, 32, 1, 8192, 256) == 1
+    assert dkdv_heads_per_slice(1, 32, 4, 8192, 256) == 4     # 64 key blocks x 8 kv heads = 512 workgroups
+    assert dkdv_heads_per_slice(1, 32, 8, 8192, 256) == 4     # whole groups would leave 256 workgroups
+    assert dkdv_heads_per_slice(1, 8, 8, 1024, 256) == 1      # tiny launch: one slice per query head
+    for args in [(2, 40, 5, 3000, 256), (1, 6, 6, 70000, 304), (3, 16, 2, 100, 256)]:
+        c = dkdv_heads_per_slice(*args)
+        assert 1 <= c <= args[2] and args[2] % c == 0
+
+
 def test_paged_launch_choice():
     # (num_seqs, kv heads, group, head size, max context, compute units)
     assert choose_launch(64, 8, 4, 128, 8192, 256) == ("balanced", 512)

@@ -60,13 +60,11 @@ def test_flash_forward_backward_total(lib, B, H, Hk, M, N, D, causal, dtype, bth
     _abi.fa_total_attn(lib, qd, kd, lse, tot, causal, sc)
     delta = torch.full((B, H, M), float("nan"))
     _abi.fa_bwd_delta(lib, o, do, delta)
-    dk = torch.full((B, H, N, D), float("nan"), dtype=dtype)
-    dv = torch.full((B, H, N, D), float("nan"), dtype=dtype)
+    dk = torch.full((B, Hk, N, D), float("nan"), dtype=dtype)   # group-summed by the kernel
+    dv = torch.full((B, Hk, N, D), float("nan"), dtype=dtype)
     dq = torch.full((B, H, M, D), float("nan"), dtype=dtype)
     _abi.fa_bwd_dkdv(lib, qd, kd, vd, do, lse, delta, dk, dv, causal, sc)
     _abi.fa_bwd_dq(lib, qd, kd, vd, do, lse, delta, dq, causal, sc)
-    g = H // Hk
-    dk, dv = dk.reshape(B, Hk, g, N, D).sum(2), dv.reshape(B, Hk, g, N, D).sum(2)
 
     ref = flash_attention(q, k, v, causal, upcast=True, return_log_normalizer=True, return_total_attention=True)
     same = flash_attention(q, k, v, causal, upcast=False, return_log_normalizer=True, return_total_attention=True)
@@ -107,8 +105,8 @@ def test_flash_backward_with_stored_ds(lib, B, H, Hk, M, N, D, causal, dtype, bt
     _abi.fa_fwd(lib, qd, kd, vd, o, lse, causal, sc)
     delta = torch.full((B, H, M), float("nan"))
     _abi.fa_bwd_delta(lib, o, do, delta)
-    dk = torch.full((B, H, N, D), float("nan"), dtype=dtype)
-    dv = torch.full((B, H, N, D), float("nan"), dtype=dtype)
+    dk = torch.full((B, Hk, N, D), float("nan"), dtype=dtype)   # group-summed by the kernel
+    dv = torch.full((B, Hk, N, D), float("nan"), dtype=dtype)
     dq = torch.full((B, H, M, D), float("nan"), dtype=dtype)
     mib = lib.fa_bwd_ds_workspace_mib(B, H, M, N)
     assert mib > 0
@@ -121,8 +119,6 @@ def test_flash_backward_with_stored_ds(lib, B, H, Hk, M, N, D, causal, dtype, bt
     _abi.fa_bwd_dq(lib, qd, kd, vd, do, lse, delta, dq_plain, causal, sc)
     assert torch.equal(dk, dk_plain) and torch.equal(dv, dv_plain)
     assert not torch.isnan(dq).any()
-    g = H // Hk
-    dk, dv = dk.reshape(B, Hk, g, N, D).sum(2), dv.reshape(B, Hk, g, N, D).sum(2)
     ref = flash_attention(q, k, v, causal, upcast=True)
     same = flash_attention(q, k, v, causal, upcast=False)
     g_ref = torch.autograd.grad(ref, (q, k, v), do)
