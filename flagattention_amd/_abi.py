@@ -67,11 +67,19 @@ def kernel_ready(t):
     return t if is_kernel_ready(t) else t.clone(memory_format=torch.contiguous_format)
 
 
-def fa_fwd(lib, q, k, v, o, lse, causal, sm_scale):
+NO_DROPOUT = (0.0, 0, 0)  # (dropout_p, seed, offset)
+
+
+def _u64(x):
+    return int(x) & 0xFFFFFFFFFFFFFFFF
+
+
+def fa_fwd(lib, q, k, v, o, lse, causal, sm_scale, dropout=NO_DROPOUT):
     B, H, M, D = q.shape
     Hk, N = k.shape[1], k.shape[2]
     check(lib.fa_fwd(dtype_code(q), view4(q), view4(k), view4(v), view4(o), ptr(lse),
-                     B, H, Hk, M, N, D, int(causal), float(sm_scale), stream_of(q)), "fa_fwd")
+                     B, H, Hk, M, N, D, int(causal), float(sm_scale), float(dropout[0]), _u64(dropout[1]),
+                     _u64(dropout[2]), stream_of(q)), "fa_fwd")
 
 
 def pw_fwd(lib, q1, k1, q2, k2, v, o, lse, w, causal, sm_scale):
@@ -95,29 +103,31 @@ def _heads_per_slice(q, dk):
     return H // slices
 
 
-def fa_bwd_dkdv(lib, q, k, v, do, lse, delta, dk, dv, causal, sm_scale):
+def fa_bwd_dkdv(lib, q, k, v, do, lse, delta, dk, dv, causal, sm_scale, dropout=NO_DROPOUT):
     B, H, M, D = q.shape
     Hk, N = k.shape[1], k.shape[2]
     check(lib.fa_bwd_dkdv(dtype_code(q), view4(q), view4(k), view4(v), view4(do), ptr(lse), ptr(delta),
                           view4(dk), view4(dv), _heads_per_slice(q, dk), B, H, Hk, M, N, D, int(causal),
-                          float(sm_scale), stream_of(q)), "fa_bwd_dkdv")
+                          float(sm_scale), float(dropout[0]), _u64(dropout[1]), _u64(dropout[2]),
+                          stream_of(q)), "fa_bwd_dkdv")
 
 
-def fa_bwd_dq(lib, q, k, v, do, lse, delta, dq, causal, sm_scale):
+def fa_bwd_dq(lib, q, k, v, do, lse, delta, dq, causal, sm_scale, dropout=NO_DROPOUT):
     B, H, M, D = q.shape
     Hk, N = k.shape[1], k.shape[2]
     check(lib.fa_bwd_dq(dtype_code(q), view4(q), view4(k), view4(v), view4(do), ptr(lse), ptr(delta),
-                        view4(dq), B, H, Hk, M, N, D, int(causal), float(sm_scale), stream_of(q)),
-          "fa_bwd_dq")
+                        view4(dq), B, H, Hk, M, N, D, int(causal), float(sm_scale), float(dropout[0]),
+                        _u64(dropout[1]), _u64(dropout[2]), stream_of(q)), "fa_bwd_dq")
 
 
-def fa_bwd_dkdv_ds(lib, q, k, v, do, lse, delta, dk, dv, ds, causal, sm_scale):
+def fa_bwd_dkdv_ds(lib, q, k, v, do, lse, delta, dk, dv, ds, causal, sm_scale, dropout=NO_DROPOUT):
     B, H, M, D = q.shape
     Hk, N = k.shape[1], k.shape[2]
     check(lib.fa_bwd_dkdv_ds(dtype_code(q), view4(q), view4(k), view4(v), view4(do), ptr(lse), ptr(delta),
                              view4(dk), view4(dv), _heads_per_slice(q, dk), ptr(ds),
                              ds.numel() * ds.element_size(), B, H, Hk, M, N, D, int(causal),
-                             float(sm_scale), stream_of(q)), "fa_bwd_dkdv_ds")
+                             float(sm_scale), float(dropout[0]), _u64(dropout[1]), _u64(dropout[2]),
+                             stream_of(q)), "fa_bwd_dkdv_ds")
 
 
 def fa_bwd_dq_from_ds(lib, k, ds, dq, causal, sm_scale):

@@ -16,19 +16,20 @@ class View4(ctypes.Structure):
                 ("stride_h", ctypes.c_int64), ("stride_t", ctypes.c_int64)]
 
 
-_i, _f, _p, _i64 = ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_int64
+_i, _f, _p, _i64, _u64 = ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_int64, ctypes.c_uint64
 _v = ctypes.POINTER(View4)
 
 # name -> argument types, in the order of include/flagattn.h
 SIGNATURES = {
     "fa_version": [],
     "fa_num_cus": [],
-    "fa_fwd": [_i, _v, _v, _v, _v, _p, _i, _i, _i, _i, _i, _i, _i, _f, _p],
+    "fa_fwd": [_i, _v, _v, _v, _v, _p, _i, _i, _i, _i, _i, _i, _i, _f, _f, _u64, _u64, _p],
     "fa_bwd_delta": [_i, _v, _v, _p, _i, _i, _i, _i, _p],
-    "fa_bwd_dkdv": [_i, _v, _v, _v, _v, _p, _p, _v, _v, _i, _i, _i, _i, _i, _i, _i, _i, _f, _p],
-    "fa_bwd_dq": [_i, _v, _v, _v, _v, _p, _p, _v, _i, _i, _i, _i, _i, _i, _i, _f, _p],
+    "fa_bwd_dkdv": [_i, _v, _v, _v, _v, _p, _p, _v, _v, _i, _i, _i, _i, _i, _i, _i, _i, _f, _f, _u64, _u64, _p],
+    "fa_bwd_dq": [_i, _v, _v, _v, _v, _p, _p, _v, _i, _i, _i, _i, _i, _i, _i, _f, _f, _u64, _u64, _p],
     "fa_bwd_ds_workspace_mib": [_i, _i, _i, _i],
-    "fa_bwd_dkdv_ds": [_i, _v, _v, _v, _v, _p, _p, _v, _v, _i, _p, _i64, _i, _i, _i, _i, _i, _i, _i, _f, _p],
+    "fa_bwd_dkdv_ds": [_i, _v, _v, _v, _v, _p, _p, _v, _v, _i, _p, _i64, _i, _i, _i, _i, _i, _i, _i, _f, _f, _u64,
+                       _u64, _p],
     "fa_bwd_dq_from_ds": [_i, _v, _p, _i64, _v, _i, _i, _i, _i, _i, _i, _i, _f, _p],
     "fa_total_attn": [_i, _v, _v, _p, _p, _i, _i, _i, _i, _i, _i, _i, _f, _p],
     "fa_splitkv_fwd": [_i, _v, _v, _v, _p, _p, _i, _i, _i, _i, _i, _i, _i, _f, _i, _i, _p],

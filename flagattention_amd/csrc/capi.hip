@@ -44,7 +44,7 @@ int fa_num_cus(void) {
 
 int fa_fwd(int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v, const fa_view4* o,
            float* lse, int B, int H, int Hk, int M, int N, int D, int causal, float sm_scale,
-           void* stream) {
+           float dropout_p, uint64_t seed, uint64_t offset, void* stream) {
   if (!view_ok(q) || !view_ok(k) || !view_ok(v) || !view_ok(o) || !lse) return FA_ERR_BAD_ARGUMENT;
   if (!head_dim_ok(D)) return FA_ERR_UNSUPPORTED;
   if (Hk <= 0 || H % Hk) return FA_ERR_BAD_ARGUMENT;
@@ -54,6 +54,7 @@ int fa_fwd(int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v, c
   p.B = B; p.H = H; p.M = M; p.N = N; p.D = D;
   p.group = H / Hk;
   p.causal = causal; p.w = 0; p.sm_scale = sm_scale; p.dtype = dtype;
+  p.dropout_p = dropout_p; p.seed = seed; p.offset = offset;
   return fa::run_fwd(p, false, (hipStream_t)stream);
 }
 
@@ -100,24 +101,27 @@ static int fill_bwd(fa::BwdParams& p, int dtype, const fa_view4* q, const fa_vie
 int fa_bwd_dkdv(int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v,
                 const fa_view4* dout, const float* lse, const float* delta, const fa_view4* dk,
                 const fa_view4* dv, int heads_per_slice, int B, int H, int Hk, int M, int N, int D,
-                int causal, float sm_scale, void* stream) {
+                int causal, float sm_scale, float dropout_p, uint64_t seed, uint64_t offset, void* stream) {
   fa::BwdParams p = {};
   int rc = fill_bwd(p, dtype, q, k, v, dout, lse, delta, B, H, Hk, M, N, D, causal, sm_scale);
   if (rc) return rc;
   if (!view_ok(dk) || !view_ok(dv)) return FA_ERR_BAD_ARGUMENT;
   p.dk = to_view(dk); p.dv = to_view(dv);
   p.chunk = heads_per_slice;
+  p.dropout_p = dropout_p; p.seed = seed; p.offset = offset;
   return fa::run_bwd_dkdv(p, false, (hipStream_t)stream);
 }
 
 int fa_bwd_dq(int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v,
               const fa_view4* dout, const float* lse, const float* delta, const fa_view4* dq, int B,
-              int H, int Hk, int M, int N, int D, int causal, float sm_scale, void* stream) {
+              int H, int Hk, int M, int N, int D, int causal, float sm_scale, float dropout_p,
+              uint64_t seed, uint64_t offset, void* stream) {
   fa::BwdParams p = {};
   int rc = fill_bwd(p, dtype, q, k, v, dout, lse, delta, B, H, Hk, M, N, D, causal, sm_scale);
   if (rc) return rc;
   if (!view_ok(dq)) return FA_ERR_BAD_ARGUMENT;
   p.dq = to_view(dq);
+  p.dropout_p = dropout_p; p.seed = seed; p.offset = offset;
   return fa::run_bwd_dq(p, false, (hipStream_t)stream);
 }
 
@@ -130,7 +134,8 @@ int fa_bwd_ds_workspace_mib(int B, int H, int M, int N) {
 int fa_bwd_dkdv_ds(int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v,
                    const fa_view4* dout, const float* lse, const float* delta, const fa_view4* dk,
                    const fa_view4* dv, int heads_per_slice, void* ds_workspace, int64_t ds_workspace_bytes,
-                   int B, int H, int Hk, int M, int N, int D, int causal, float sm_scale, void* stream) {
+                   int B, int H, int Hk, int M, int N, int D, int causal, float sm_scale, float dropout_p,
+                   uint64_t seed, uint64_t offset, void* stream) {
   fa::BwdParams p = {};
   int rc = fill_bwd(p, dtype, q, k, v, dout, lse, delta, B, H, Hk, M, N, D, causal, sm_scale);
   if (rc) return rc;
@@ -140,6 +145,7 @@ int fa_bwd_dkdv_ds(int dtype, const fa_view4* q, const fa_view4* k, const fa_vie
     return FA_ERR_BAD_ARGUMENT;
   p.dk = to_view(dk); p.dv = to_view(dv);
   p.chunk = heads_per_slice;
+  p.dropout_p = dropout_p; p.seed = seed; p.offset = offset;
   p.ds = ds_workspace;
   return fa::run_bwd_dkdv_ds(p, (hipStream_t)stream);
 }

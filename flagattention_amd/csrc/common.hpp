@@ -134,6 +134,37 @@ FA_DEVICE typename hw::Elem<T>::v8 pack_half_block(const f32x16& s, int c) {
 }
 
 // ---------------------------------------------------------------------------------------------
+// dropout mask
+// ---------------------------------------------------------------------------------------------
+// The reference draws one number per score element with Triton's tl.rand(seed, offs, n_rounds=6)
+// (src/flag_attn/flash.py:367-371, 454-457): Philox-4x32 with counter (lo(c), hi(c), 0, 0),
+// c = offset + ((b * H + h) * M + m) * N + n, key (lo(seed), hi(seed)), 6 rounds, first output word;
+// the word, read as int32 with negative values folded by -x - 1, times 4.6566127342e-10 is the
+// uniform number, and the probability is kept when it exceeds dropout_p.
+FA_DEVICE uint32_t philox6_first_word(uint32_t c0, uint32_t c1, uint32_t k0, uint32_t k1) {
+  uint32_t c2 = 0u, c3 = 0u;
+#pragma unroll
+  for (int round = 0; round < 6; ++round) {
+    const uint64_t p0 = (uint64_t)0xD2511F53u * c0, p1 = (uint64_t)0xCD9E8D57u * c2;
+    const uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0, n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+    c1 = (uint32_t)p1;
+    c3 = (uint32_t)p0;
+    c0 = n0;
+    c2 = n2;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+  return c0;
+}
+FA_DEVICE bool dropout_keeps(uint64_t counter, uint64_t seed, float dropout_p) {
+  const uint32_t x = philox6_first_word((uint32_t)counter, (uint32_t)(counter >> 32), (uint32_t)seed,
+                                        (uint32_t)(seed >> 32));
+  int32_t v = (int32_t)x;
+  v = v < 0 ? ~v : v;  // -v - 1
+  return (float)v * 4.6566127342e-10f > dropout_p;
+}
+
+// ---------------------------------------------------------------------------------------------
 // launch
 // ---------------------------------------------------------------------------------------------
 #ifdef FLAGATTN_HOST_SIM

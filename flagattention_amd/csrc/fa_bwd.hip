@@ -90,9 +90,17 @@ struct KvCfg {
 // fa_bwd_dq_from_ds_kernel, one 2 KB chunk per 32 x 32 block in the order the MFMA result holds it:
 // chunk[c][lane] = 8 elements, queries 16c + 8g + 4(lane / 32) + e at position 4g + e, key lane % 32.
 // Chunks are indexed (batch * H + head, key block, query block); both counts padded to 4.
-template <class T, int D, bool PW, bool DS = false>
-FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (KvCfg<T, D, PW>::WAVES_PER_SIMD)) fa_bwd_dkdv_kernel(BwdParams p) {
+//
+// DROP: dropout as in the reference (flash.py:697-721): dV takes the masked P and is scaled by
+// 1 / (1 - dropout_p); dP is masked and scaled likewise; dS = P (dP - delta) with the unmasked P.
+//
+// GROUPED: the workgroup walks more than one query head (see below); a separate instantiation,
+// because the extra loop level costs the single-head kernel 10 % through register allocation alone.
+template <class T, int D, bool PW, bool DS = false, bool DROP = false, bool GROUPED = false>
+FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PER_SIMD)) fa_bwd_dkdv_kernel(BwdParams p) {
+  static_assert(!(GROUPED && (PW || DROP)), "grouped accumulation is built for plain attention without dropout");
   static_assert(!(PW && DS), "the dS workspace is only defined for plain flash attention");
+  static_assert(!(PW && DROP), "piecewise attention has no dropout");
   using C = KvCfg<T, D, PW>;
   using V8 = typename hw::Elem<T>::v8;
   FA_LDS_DECL(smem);
@@ -103,7 +111,7 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (KvCfg<T, D, PW>::WAVES_PER_SIMD)) fa
   // the chunk one after the other and accumulates their dK / dV in the same registers, so the sum
   // over the chunk costs nothing.  chunk = group gives dK/dV per kv head; smaller chunks (more
   // workgroups, for launches that would not fill the device) leave group / chunk slices to add.
-  const int chunk = p.chunk > 0 ? p.chunk : p.group;
+  const int chunk = GROUPED ? (p.chunk > 0 ? p.chunk : p.group) : 1;
   const TileId wg = tile_of_workgroup(p.H / chunk, p.B);  // key blocks in ascending order: most queries first
   const int slice = wg.head, batch = wg.batch;             // output slice = chunk index
   const int hk = slice * chunk / p.group;
@@ -179,6 +187,8 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (KvCfg<T, D, PW>::WAVES_PER_SIMD)) fa
   };
 
   const float c2 = p.sm_scale * kLog2e;
+  const float rp = DROP ? 1.f / (1.f - p.dropout_p) : 1.f;
+  uint64_t drop_col = 0;  // dropout counter of (query 0, my_n) of the current head
 
   // result block (keys x D): D along lanes, keys along registers
   auto store_keys = [&](const f32x16* acc, const View4& dst, float scale) {
@@ -207,6 +217,7 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (KvCfg<T, D, PW>::WAVES_PER_SIMD)) fa
     const int64_t nqb = 4 * (int64_t)cdiv(M, 128), nkb = 4 * (int64_t)cdiv(N, 128);
     ds_row = (T*)p.ds + ((((int64_t)batch * p.H + head) * nkb + (n0 / 32 + wave)) * nqb) * 1024 + lane * 8;
   }
+  if (DROP) drop_col = p.offset + ((uint64_t)batch * p.H + head) * M * (uint64_t)N + (uint64_t)(my_n < N ? my_n : 0);
 #pragma unroll
   for (int ph = 0; ph < (PW ? 2 : 1); ++ph) {
     far_phase = PW && ph == 1;
@@ -275,15 +286,27 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (KvCfg<T, D, PW>::WAVES_PER_SIMD)) fa
             if (PW) keep = keep && ((m + pseq - my_n >= p.w) == far_phase);
             float pv = hw::exp2_fast(fmaf(s[r], c2, -lrow[r >> 2][r & 3]));
             pv = keep ? pv : 0.f;
-            pr[r] = pv;
-            ds[r] = pv * (dp[r] - drow[r >> 2][r & 3]);
+            float pd = pv, dpv = dp[r];
+            if (DROP) {
+              const bool kd = dropout_keeps(drop_col + (uint64_t)m * N, p.seed, p.dropout_p);
+              pd = kd ? pv : 0.f;
+              dpv = kd ? dp[r] * rp : 0.f;
+            }
+            pr[r] = pd;
+            ds[r] = pv * (dpv - drow[r >> 2][r & 3]);
           }
         } else {
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
             const float pv = hw::exp2_fast(fmaf(s[r], c2, -lrow[r >> 2][r & 3]));
-            pr[r] = pv;
-            ds[r] = pv * (dp[r] - drow[r >> 2][r & 3]);
+            float pd = pv, dpv = dp[r];
+            if (DROP) {
+              const bool kd = dropout_keeps(drop_col + (uint64_t)(mr0 + block_row(r, hh)) * N, p.seed, p.dropout_p);
+              pd = kd ? pv : 0.f;
+              dpv = kd ? dp[r] * rp : 0.f;
+            }
+            pr[r] = pd;
+            ds[r] = pv * (dpv - drow[r >> 2][r & 3]);
           }
         }
 #pragma unroll
@@ -319,7 +342,7 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (KvCfg<T, D, PW>::WAVES_PER_SIMD)) fa
   }
   }
   if (!PW) store_keys(dk, p.dk, p.sm_scale);
-  store_keys(dv, p.dv, 1.f);
+  store_keys(dv, p.dv, rp);
 }
 
 // ----------------------------------------------------------------------------------- dQ ----
@@ -338,8 +361,10 @@ struct QCfg {
 
 // PW: two passes over the key tiles, as in the forward kernel -- the far keys with (q2, k2)
 // accumulating dQ2, then the near keys with (q1, k1) accumulating dQ1 in the same registers.
-template <class T, int D, bool PW>
+// DROP: dP is masked and scaled by 1 / (1 - dropout_p) before dS = P (dP - delta) (flash.py:877-890).
+template <class T, int D, bool PW, bool DROP = false>
 FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (QCfg<T, D, PW>::WAVES_PER_SIMD)) fa_bwd_dq_kernel(BwdParams p) {
+  static_assert(!(PW && DROP), "piecewise attention has no dropout");
   using C = QCfg<T, D, PW>;
   using V8 = typename hw::Elem<T>::v8;
   FA_LDS_DECL(smem);
@@ -372,6 +397,9 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (QCfg<T, D, PW>::WAVES_PER_SIMD)) fa_
   const int64_t row_off = ((int64_t)batch * p.H + head) * M + my_m;
   const float l_row = my_m < M ? p.lse[row_off] * kLog2e : __builtin_inff();
   const float d_row = my_m < M ? p.delta[row_off] : 0.f;
+  const float rp = DROP ? 1.f / (1.f - p.dropout_p) : 1.f;
+  // dropout counter of (my_m, key 0)
+  const uint64_t drop_row = DROP ? p.offset + (((uint64_t)batch * p.H + head) * M + (uint64_t)(my_m < M ? my_m : 0)) * N : 0;
 
   int hi = N;
   if (p.causal) hi = imin(N, pseq + m0 + C::BM);
@@ -486,11 +514,18 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (QCfg<T, D, PW>::WAVES_PER_SIMD)) fa_
             if (PW) keep = keep && ((my_m + pseq - n >= p.w) == far_phase);
             float pv = hw::exp2_fast(fmaf(s[r], c2, -l_row));
             pv = keep ? pv : 0.f;
-            ds[r] = pv * (dp[r] - d_row);
+            float dpv = dp[r];
+            if (DROP) dpv = dropout_keeps(drop_row + (uint64_t)n, p.seed, p.dropout_p) ? dp[r] * rp : 0.f;
+            ds[r] = pv * (dpv - d_row);
           }
         } else {
 #pragma unroll
-          for (int r = 0; r < 16; ++r) ds[r] = hw::exp2_fast(fmaf(s[r], c2, -l_row)) * (dp[r] - d_row);
+          for (int r = 0; r < 16; ++r) {
+            float dpv = dp[r];
+            if (DROP)
+              dpv = dropout_keeps(drop_row + (uint64_t)(nlo + block_row(r, hh)), p.seed, p.dropout_p) ? dp[r] * rp : 0.f;
+            ds[r] = hw::exp2_fast(fmaf(s[r], c2, -l_row)) * (dpv - d_row);
+          }
         }
 #pragma unroll
         for (int c = 0; c < 2; ++c) {
@@ -656,58 +691,74 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, 2) fa_bwd_dq_from_ds_kernel(BwdParams
 }
 
 // ------------------------------------------------------------------------------ launchers ----
-template <class T, bool PW>
+template <class T, bool PW, bool DS, bool DROP, bool GROUPED>
 static int launch_dkdv(const BwdParams& p, hipStream_t stream) {
-  dim3 grid(((p.N + 127) / 128) * (p.H / (p.chunk > 0 ? p.chunk : p.group)) * p.B, 1, 1);
+  const int chunk = GROUPED ? (p.chunk > 0 ? p.chunk : p.group) : 1;
+  dim3 grid(((p.N + 127) / 128) * (p.H / chunk) * p.B, 1, 1);
   switch (p.D) {
-    case 16: return launch(fa_bwd_dkdv_kernel<T, 16, PW>, grid, KvCfg<T, 16, PW>::LDS_BYTES, stream, p);
-    case 32: return launch(fa_bwd_dkdv_kernel<T, 32, PW>, grid, KvCfg<T, 32, PW>::LDS_BYTES, stream, p);
-    case 64: return launch(fa_bwd_dkdv_kernel<T, 64, PW>, grid, KvCfg<T, 64, PW>::LDS_BYTES, stream, p);
-    case 128: return launch(fa_bwd_dkdv_kernel<T, 128, PW>, grid, KvCfg<T, 128, PW>::LDS_BYTES, stream, p);
+    case 16: return launch(fa_bwd_dkdv_kernel<T, 16, PW, DS, DROP, GROUPED>, grid, KvCfg<T, 16, PW>::LDS_BYTES, stream, p);
+    case 32: return launch(fa_bwd_dkdv_kernel<T, 32, PW, DS, DROP, GROUPED>, grid, KvCfg<T, 32, PW>::LDS_BYTES, stream, p);
+    case 64: return launch(fa_bwd_dkdv_kernel<T, 64, PW, DS, DROP, GROUPED>, grid, KvCfg<T, 64, PW>::LDS_BYTES, stream, p);
+    case 128: return launch(fa_bwd_dkdv_kernel<T, 128, PW, DS, DROP, GROUPED>, grid, KvCfg<T, 128, PW>::LDS_BYTES, stream, p);
   }
   return kUnsupported;
 }
 
-template <class T, bool PW>
+template <class T, bool PW, bool DROP>
 static int launch_dq(const BwdParams& p, hipStream_t stream) {
   dim3 grid(((p.M + 127) / 128) * p.H * p.B, 1, 1);
   switch (p.D) {
-    case 16: return launch(fa_bwd_dq_kernel<T, 16, PW>, grid, QCfg<T, 16, PW>::LDS_BYTES, stream, p);
-    case 32: return launch(fa_bwd_dq_kernel<T, 32, PW>, grid, QCfg<T, 32, PW>::LDS_BYTES, stream, p);
-    case 64: return launch(fa_bwd_dq_kernel<T, 64, PW>, grid, QCfg<T, 64, PW>::LDS_BYTES, stream, p);
-    case 128: return launch(fa_bwd_dq_kernel<T, 128, PW>, grid, QCfg<T, 128, PW>::LDS_BYTES, stream, p);
+    case 16: return launch(fa_bwd_dq_kernel<T, 16, PW, DROP>, grid, QCfg<T, 16, PW>::LDS_BYTES, stream, p);
+    case 32: return launch(fa_bwd_dq_kernel<T, 32, PW, DROP>, grid, QCfg<T, 32, PW>::LDS_BYTES, stream, p);
+    case 64: return launch(fa_bwd_dq_kernel<T, 64, PW, DROP>, grid, QCfg<T, 64, PW>::LDS_BYTES, stream, p);
+    case 128: return launch(fa_bwd_dq_kernel<T, 128, PW, DROP>, grid, QCfg<T, 128, PW>::LDS_BYTES, stream, p);
   }
   return kUnsupported;
 }
 
+static bool bwd_args_ok(const BwdParams& p, bool piecewise) {
+  if (p.B <= 0 || p.H <= 0 || p.M <= 0 || p.N <= 0 || p.group <= 0) return false;
+  if (p.chunk < 0 || (p.chunk > 0 && p.group % p.chunk)) return false;
+  if (!(p.dropout_p >= 0.f && p.dropout_p < 1.f) || (piecewise && p.dropout_p > 0.f)) return false;
+  return true;
+}
+
+// summed dK/dV slices are built for plain attention without dropout
+static bool dkdv_chunk_ok(const BwdParams& p, bool piecewise) {
+  const int chunk = p.chunk > 0 ? p.chunk : p.group;
+  return chunk == 1 || !(piecewise || p.dropout_p > 0.f);
+}
+
+template <class T>
+static int dispatch_dkdv(const BwdParams& p, bool piecewise, bool keep_ds, hipStream_t stream) {
+  if (piecewise) return launch_dkdv<T, true, false, false, false>(p, stream);
+  const bool drop = p.dropout_p > 0.f;
+  const bool grouped = (p.chunk > 0 ? p.chunk : p.group) > 1;
+  if (keep_ds) {
+    if (drop) return launch_dkdv<T, false, true, true, false>(p, stream);
+    return grouped ? launch_dkdv<T, false, true, false, true>(p, stream) : launch_dkdv<T, false, true, false, false>(p, stream);
+  }
+  if (drop) return launch_dkdv<T, false, false, true, false>(p, stream);
+  return grouped ? launch_dkdv<T, false, false, false, true>(p, stream) : launch_dkdv<T, false, false, false, false>(p, stream);
+}
+
+template <class T>
+static int dispatch_dq(const BwdParams& p, bool piecewise, hipStream_t stream) {
+  if (piecewise) return launch_dq<T, true, false>(p, stream);
+  return p.dropout_p > 0.f ? launch_dq<T, false, true>(p, stream) : launch_dq<T, false, false>(p, stream);
+}
+
 int run_bwd_dkdv(const BwdParams& p, bool piecewise, hipStream_t stream) {
-  if (p.B <= 0 || p.H <= 0 || p.M <= 0 || p.N <= 0 || p.group <= 0) return kBadArgument;
-  if (p.chunk < 0 || (p.chunk > 0 && p.group % p.chunk)) return kBadArgument;
-  if (p.dtype == kDtypeF16)
-    return piecewise ? launch_dkdv<hw::half_t, true>(p, stream) : launch_dkdv<hw::half_t, false>(p, stream);
-  if (p.dtype == kDtypeBF16)
-    return piecewise ? launch_dkdv<hw::bf16_t, true>(p, stream) : launch_dkdv<hw::bf16_t, false>(p, stream);
+  if (!bwd_args_ok(p, piecewise) || !dkdv_chunk_ok(p, piecewise)) return kBadArgument;
+  if (p.dtype == kDtypeF16) return dispatch_dkdv<hw::half_t>(p, piecewise, false, stream);
+  if (p.dtype == kDtypeBF16) return dispatch_dkdv<hw::bf16_t>(p, piecewise, false, stream);
   return kUnsupported;
 }
 
 int run_bwd_dq(const BwdParams& p, bool piecewise, hipStream_t stream) {
-  if (p.B <= 0 || p.H <= 0 || p.M <= 0 || p.N <= 0 || p.group <= 0) return kBadArgument;
-  if (p.dtype == kDtypeF16)
-    return piecewise ? launch_dq<hw::half_t, true>(p, stream) : launch_dq<hw::half_t, false>(p, stream);
-  if (p.dtype == kDtypeBF16)
-    return piecewise ? launch_dq<hw::bf16_t, true>(p, stream) : launch_dq<hw::bf16_t, false>(p, stream);
-  return kUnsupported;
-}
-
-template <class T>
-static int launch_dkdv_ds(const BwdParams& p, hipStream_t stream) {
-  dim3 grid(((p.N + 127) / 128) * (p.H / (p.chunk > 0 ? p.chunk : p.group)) * p.B, 1, 1);
-  switch (p.D) {
-    case 16: return launch(fa_bwd_dkdv_kernel<T, 16, false, true>, grid, KvCfg<T, 16, false>::LDS_BYTES, stream, p);
-    case 32: return launch(fa_bwd_dkdv_kernel<T, 32, false, true>, grid, KvCfg<T, 32, false>::LDS_BYTES, stream, p);
-    case 64: return launch(fa_bwd_dkdv_kernel<T, 64, false, true>, grid, KvCfg<T, 64, false>::LDS_BYTES, stream, p);
-    case 128: return launch(fa_bwd_dkdv_kernel<T, 128, false, true>, grid, KvCfg<T, 128, false>::LDS_BYTES, stream, p);
-  }
+  if (!bwd_args_ok(p, piecewise)) return kBadArgument;
+  if (p.dtype == kDtypeF16) return dispatch_dq<hw::half_t>(p, piecewise, stream);
+  if (p.dtype == kDtypeBF16) return dispatch_dq<hw::bf16_t>(p, piecewise, stream);
   return kUnsupported;
 }
 
@@ -728,10 +779,9 @@ int64_t bwd_ds_workspace_bytes(int B, int H, int M, int N) {
 }
 
 int run_bwd_dkdv_ds(const BwdParams& p, hipStream_t stream) {
-  if (p.B <= 0 || p.H <= 0 || p.M <= 0 || p.N <= 0 || p.group <= 0 || !p.ds) return kBadArgument;
-  if (p.chunk < 0 || (p.chunk > 0 && p.group % p.chunk)) return kBadArgument;
-  if (p.dtype == kDtypeF16) return launch_dkdv_ds<hw::half_t>(p, stream);
-  if (p.dtype == kDtypeBF16) return launch_dkdv_ds<hw::bf16_t>(p, stream);
+  if (!bwd_args_ok(p, false) || !dkdv_chunk_ok(p, false) || !p.ds) return kBadArgument;
+  if (p.dtype == kDtypeF16) return dispatch_dkdv<hw::half_t>(p, false, true, stream);
+  if (p.dtype == kDtypeBF16) return dispatch_dkdv<hw::bf16_t>(p, false, true, stream);
   return kUnsupported;
 }
 

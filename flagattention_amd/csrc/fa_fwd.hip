@@ -32,8 +32,11 @@ struct FwdCfg {
   static constexpr size_t LDS_BYTES = 2 * STAGE * sizeof(T);
 };
 
-template <class T, int D, bool PW>
+// DROP: dropout as in the reference (flash.py:450-457, 479-482): the row sum is taken before the mask,
+// dropped probabilities do not enter the second product, the output is scaled by 1 / (1 - dropout_p).
+template <class T, int D, bool PW, bool DROP = false>
 FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (FwdCfg<T, D, PW>::WAVES_PER_SIMD)) fa_fwd_kernel(FwdParams p) {
+  static_assert(!(PW && DROP), "piecewise attention has no dropout");
   using C = FwdCfg<T, D, PW>;
   using V8 = typename hw::Elem<T>::v8;
   FA_LDS_DECL(smem);
@@ -77,6 +80,8 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (FwdCfg<T, D, PW>::WAVES_PER_SIMD)) f
   }
 
   const float c2 = p.sm_scale * kLog2e;
+  // dropout counter of (my_m, key 0)
+  const uint64_t drop_row = DROP ? p.offset + (((uint64_t)batch * p.H + head) * M + (uint64_t)(my_m < M ? my_m : 0)) * N : 0;
   float m_i = neg_inf(), l_i = 0.f;
   f32x16 oacc[C::DV / 32];
 #pragma unroll
@@ -163,8 +168,9 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (FwdCfg<T, D, PW>::WAVES_PER_SIMD)) f
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         float e = hw::exp2_fast(fmaf(s[nb][r], c2, shift));
-        s[nb][r] = e;
         psum += e;
+        if (DROP) e = dropout_keeps(drop_row + (uint64_t)(n0 + nb * 32 + block_row(r, hh)), p.seed, p.dropout_p) ? e : 0.f;
+        s[nb][r] = e;
       }
     // The accumulators are rescaled only when some row of the wavefront raised its maximum;
     // after the first few tiles that is rare.
@@ -227,7 +233,7 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (FwdCfg<T, D, PW>::WAVES_PER_SIMD)) f
   // ---- epilogue: O = acc / l, L = m * scale + ln(l); rows that saw no key give O = 0, L = -inf ----
   const float l_tot = l_i + hw::xor32(l_i);
   const bool empty = !(l_tot > 0.f);
-  const float inv = empty ? 0.f : 1.f / l_tot;
+  const float inv = empty ? 0.f : (DROP ? 1.f / ((1.f - p.dropout_p) * l_tot) : 1.f / l_tot);
   if (my_m < M) {
     T* ob = (T*)p.o.ptr + batch * p.o.sb + head * p.o.sh + (int64_t)my_m * p.o.st;
 #pragma unroll
@@ -247,24 +253,29 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (FwdCfg<T, D, PW>::WAVES_PER_SIMD)) f
   }
 }
 
-template <class T, bool PW>
+template <class T, bool PW, bool DROP>
 static int launch_fwd(const FwdParams& p, hipStream_t stream) {
   dim3 grid(((p.M + 127) / 128) * p.H * p.B, 1, 1);
   switch (p.D) {
-    case 16: return launch(fa_fwd_kernel<T, 16, PW>, grid, FwdCfg<T, 16, PW>::LDS_BYTES, stream, p);
-    case 32: return launch(fa_fwd_kernel<T, 32, PW>, grid, FwdCfg<T, 32, PW>::LDS_BYTES, stream, p);
-    case 64: return launch(fa_fwd_kernel<T, 64, PW>, grid, FwdCfg<T, 64, PW>::LDS_BYTES, stream, p);
-    case 128: return launch(fa_fwd_kernel<T, 128, PW>, grid, FwdCfg<T, 128, PW>::LDS_BYTES, stream, p);
+    case 16: return launch(fa_fwd_kernel<T, 16, PW, DROP>, grid, FwdCfg<T, 16, PW>::LDS_BYTES, stream, p);
+    case 32: return launch(fa_fwd_kernel<T, 32, PW, DROP>, grid, FwdCfg<T, 32, PW>::LDS_BYTES, stream, p);
+    case 64: return launch(fa_fwd_kernel<T, 64, PW, DROP>, grid, FwdCfg<T, 64, PW>::LDS_BYTES, stream, p);
+    case 128: return launch(fa_fwd_kernel<T, 128, PW, DROP>, grid, FwdCfg<T, 128, PW>::LDS_BYTES, stream, p);
   }
   return kUnsupported;
 }
 
+template <class T>
+static int dispatch_fwd(const FwdParams& p, bool piecewise, hipStream_t stream) {
+  if (piecewise) return launch_fwd<T, true, false>(p, stream);
+  return p.dropout_p > 0.f ? launch_fwd<T, false, true>(p, stream) : launch_fwd<T, false, false>(p, stream);
+}
+
 int run_fwd(const FwdParams& p, bool piecewise, hipStream_t stream) {
   if (p.B <= 0 || p.H <= 0 || p.M <= 0 || p.N < 0 || p.group <= 0) return kBadArgument;
-  if (p.dtype == kDtypeF16)
-    return piecewise ? launch_fwd<hw::half_t, true>(p, stream) : launch_fwd<hw::half_t, false>(p, stream);
-  if (p.dtype == kDtypeBF16)
-    return piecewise ? launch_fwd<hw::bf16_t, true>(p, stream) : launch_fwd<hw::bf16_t, false>(p, stream);
+  if (!(p.dropout_p >= 0.f && p.dropout_p < 1.f) || (piecewise && p.dropout_p > 0.f)) return kBadArgument;
+  if (p.dtype == kDtypeF16) return dispatch_fwd<hw::half_t>(p, piecewise, stream);
+  if (p.dtype == kDtypeBF16) return dispatch_fwd<hw::bf16_t>(p, piecewise, stream);
   return kUnsupported;
 }
 

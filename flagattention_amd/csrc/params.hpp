@@ -21,6 +21,8 @@ struct FwdParams {
   int w;                  // piecewise distance threshold
   float sm_scale;
   int dtype;
+  float dropout_p;        // 0 = no dropout; otherwise the mask is drawn from (seed, offset)
+  uint64_t seed, offset;
 };
 
 struct BwdParams {
@@ -36,6 +38,8 @@ struct BwdParams {
   int w;
   float sm_scale;
   int dtype;
+  float dropout_p;
+  uint64_t seed, offset;
 };
 
 struct TotalParams {

@@ -46,8 +46,7 @@ class FlashAttention(torch.autograd.Function):
         Hk, Hv = k.shape[1], v.shape[1]
         assert Hk == Hv, "num of heads in k and v should be equal"
         assert H % Hk == 0, "number of heads in q must be a multiple of that in k & v"
-        if dropout_p > 0:
-            raise NotImplementedError("dropout is not implemented by the gfx950 kernels yet")
+        assert 0.0 <= dropout_p < 1.0, "dropout_p must be in [0, 1)"
         if sm_scale is None:
             sm_scale = 1.0 / math.sqrt(D)
 
@@ -56,15 +55,23 @@ class FlashAttention(torch.autograd.Function):
 
         with torch.cuda.device(q.device):
             num_cus = lib.fa_num_cus()
+            is_dropout = dropout_p > 0
+            if is_dropout:   # one Philox counter value per score element (flash.py:52-57)
+                seed, offset = philox_seed_offset(B * H * M * N, q.device)
+            else:
+                seed, offset = 0, 0
+            dropout = (dropout_p, seed, offset)
             splits = num_splits_heuristic(B, H, M, N, SPLIT_BLOCK_M, SPLIT_BLOCK_N, num_cus, 128)
-            if splits > 1 or (M <= DECODE_MAX_ROWS and N >= 1024):
+            if splits > 1:
+                assert not is_dropout, "Cannot apply dropout with splitkv."   # as flash.py:89
+            if splits > 1 or (M <= DECODE_MAX_ROWS and N >= 1024 and not is_dropout):
                 o, L = split_kv_forward(lib, q, k, v, causal, sm_scale, splits)
             else:
                 o = torch.empty_like(q)
                 if not _abi.is_kernel_ready(o):
                     o = torch.empty(q.shape, dtype=q.dtype, device=q.device)
                 L = torch.empty((B, H, M), device=q.device, dtype=torch.float32)
-                _abi.fa_fwd(lib, q, k, v, o, L, causal, sm_scale)
+                _abi.fa_fwd(lib, q, k, v, o, L, causal, sm_scale, dropout)
             tot_attn = None
             if return_total_attention:
                 tot_attn = _total_attention(lib, q, k, L, causal, sm_scale)
@@ -72,18 +79,20 @@ class FlashAttention(torch.autograd.Function):
         ctx.save_for_backward(q, k, v, o, L)
         ctx.sm_scale = sm_scale
         ctx.causal = causal
+        ctx.dropout = dropout
 
         if return_log_normalizer or return_total_attention or return_seed_offset:
             return (o,
                     L if return_log_normalizer else None,
                     tot_attn if return_total_attention else None,
-                    None, None)
+                    seed if is_dropout and return_seed_offset else None,
+                    offset if is_dropout and return_seed_offset else None)
         return o
 
     @staticmethod
     def backward(ctx, do, *ignored):
         q, k, v, o, L = ctx.saved_tensors
-        sm_scale, causal = ctx.sm_scale, ctx.causal
+        sm_scale, causal, dropout = ctx.sm_scale, ctx.causal, ctx.dropout
         B, H, M, D = q.shape
         N, Hk = k.shape[2], k.shape[1]
         group = H // Hk
@@ -94,21 +103,23 @@ class FlashAttention(torch.autograd.Function):
             _abi.fa_bwd_delta(lib, o, do, delta)
             # dK/dV come out summed over each kv head's group of query heads (flash.py:205-206,250-251
             # of the reference produce one slice per query head and reduce afterwards)
-            chunk = dkdv_heads_per_slice(B, H, group, N, lib.fa_num_cus())
+            # the kernels that sum query heads are built without dropout
+            chunk = 1 if dropout[0] > 0 else dkdv_heads_per_slice(B, H, group, N, lib.fa_num_cus())
             slices = H // chunk
             dk = torch.empty((B, slices, N, D), dtype=k.dtype, device=q.device)
             dv = torch.empty((B, slices, N, D), dtype=v.dtype, device=q.device)
             dq = torch.empty((B, H, M, D), dtype=q.dtype, device=q.device)
             heads = ds_heads_per_launch(lib, B, H, group, M, N, D)
             if heads == 0:
-                _abi.fa_bwd_dkdv(lib, q, k, v, do, L, delta, dk, dv, causal, sm_scale)
-                _abi.fa_bwd_dq(lib, q, k, v, do, L, delta, dq, causal, sm_scale)
+                _abi.fa_bwd_dkdv(lib, q, k, v, do, L, delta, dk, dv, causal, sm_scale, dropout)
+                _abi.fa_bwd_dq(lib, q, k, v, do, L, delta, dq, causal, sm_scale, dropout)
             elif heads >= B * H:
                 ds = _ds_workspace(lib, q.device, B, H, M, N)
-                _abi.fa_bwd_dkdv_ds(lib, q, k, v, do, L, delta, dk, dv, ds, causal, sm_scale)
+                _abi.fa_bwd_dkdv_ds(lib, q, k, v, do, L, delta, dk, dv, ds, causal, sm_scale, dropout)
                 _abi.fa_bwd_dq_from_ds(lib, k, ds, dq, causal, sm_scale)
             else:
-                # bounded workspace: one batch entry and `heads` query heads at a time
+                # bounded workspace: one batch entry and `heads` query heads at a time; the dropout
+                # counter of a slice starts where the slice starts in the (B, H, M, N) score tensor
                 heads = min(heads, H)
                 ds = _ds_workspace(lib, q.device, 1, heads, M, N)
                 for b in range(B):
@@ -117,13 +128,28 @@ class FlashAttention(torch.autograd.Function):
                         hs, ks = slice(h0, h1), slice(h0 // group, -(-h1 // group))
                         ss = slice(h0 // chunk, h1 // chunk)
                         bs = slice(b, b + 1)
+                        drop = (dropout[0], dropout[1], dropout[2] + (b * H + h0) * M * N)
                         _abi.fa_bwd_dkdv_ds(lib, q[bs, hs], k[bs, ks], v[bs, ks], do[bs, hs], L[bs, hs],
-                                            delta[bs, hs], dk[bs, ss], dv[bs, ss], ds, causal, sm_scale)
+                                            delta[bs, hs], dk[bs, ss], dv[bs, ss], ds, causal, sm_scale, drop)
                         _abi.fa_bwd_dq_from_ds(lib, k[bs, ks], ds, dq[bs, hs], causal, sm_scale)
             if slices > Hk:   # the kernel summed `chunk` heads of every group; add the chunks
                 dk = dk.reshape(B, Hk, slices // Hk, N, D).sum(2)
                 dv = dv.reshape(B, Hk, slices // Hk, N, D).sum(2)
         return dq, dk, dv, None, None, None, None, None, None
+
+
+def philox_seed_offset(increment, device):
+    """(seed, offset) of the device's default random generator, whose offset is then advanced by
+    ``increment`` rounded up to a multiple of 4 -- the generator state is two int64 words, seed and
+    offset, exactly as ``src/flag_attn/dropout.py:5-16`` of the reference reads and advances it."""
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    gen = torch.cuda.default_generators[index]
+    state = gen.get_state()
+    words = state.view(torch.int64)
+    seed, offset = int(words[0]), int(words[1])
+    words[1] += (increment + 3) // 4 * 4
+    gen.set_state(state)
+    return seed, offset
 
 
 def dkdv_heads_per_slice(B, H, group, N, num_cus):
@@ -173,7 +199,9 @@ def attention(q, k, v, causal=False, sm_scale=None, dropout_p=0.0,
     a multiple of heads_k.  ``causal`` masks with bottom-right alignment.  Returns ``out`` or, when
     any ``return_*`` flag is set, ``(out, log_normalizer|None, total_attention|None, seed|None,
     offset|None)`` -- exactly the reference's convention (``src/flag_attn/flash.py:150-160``).
-    ``dropout_p > 0`` raises ``NotImplementedError``.
+    ``dropout_p > 0`` drops probabilities with the reference's Philox scheme (seed and offset taken from
+    the device's default generator and returned when ``return_seed_offset`` is set); it cannot be
+    combined with a shape that takes the split-KV path, as in the reference.
     """
     return FlashAttention.apply(q, k, v, causal, sm_scale, dropout_p, return_log_normalizer,
                                 return_total_attention, return_seed_offset)

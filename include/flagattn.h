@@ -47,10 +47,15 @@ int fa_num_cus(void);
  * q (B, H, M, D); k, v (B, Hk, N, D); o (B, H, M, D) written; lse (B, H, M) contiguous fp32 written
  * (natural-log normalizer of sm_scale * scores).  H % Hk == 0.  D in {16, 32, 64, 128}.
  * Causal masking is aligned bottom-right: row m sees key n iff m + N - M >= n; rows that see no key
- * get o = 0 and lse = -inf. */
+ * get o = 0 and lse = -inf.
+ * dropout_p in [0, 1), seed, offset: the reference's kernel arguments of the same names
+ * (flash.py:328-330); with dropout_p > 0 the probability of (b, h, m, n) enters the second product
+ * only if the uniform number Triton's tl.rand(seed, offset + ((b H + h) M + m) N + n, n_rounds=6) would
+ * give exceeds dropout_p, and o is scaled by 1 / (1 - dropout_p); lse is unaffected.  The backward
+ * entry points below take the same three values and must be given the forward's. */
 int fa_fwd(int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v, const fa_view4* o,
            float* lse, int B, int H, int Hk, int M, int N, int D, int causal, float sm_scale,
-           void* stream);
+           float dropout_p, uint64_t seed, uint64_t offset, void* stream);
 
 /* ----------------------------------------------------------------- flash attention, backward --
  * The reference's three launches in FlashAttention.backward, src/flag_attn/flash.py:191-249:
@@ -61,7 +66,8 @@ int fa_fwd(int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v, c
  *                  (B, H / heads_per_slice, N, D); slice s is the sum over query heads
  *                  s * heads_per_slice ... + heads_per_slice - 1 (fp32 accumulation inside the kernel).
  *                  heads_per_slice must divide H / Hk; 0 means H / Hk (one slice per kv head);
- *                  1 reproduces the reference's one slice per query head.
+ *                  1 reproduces the reference's one slice per query head and is the only value
+ *                  accepted together with dropout_p > 0.
  * fa_bwd_dq     <- `_bwd_q_kernel`   (flash.py:748-909): dq (B, H, M, D), every element written.
  * No atomics; each workgroup owns its output tile. */
 int fa_bwd_delta(int dtype, const fa_view4* o, const fa_view4* dout, float* delta, int B, int H,
@@ -69,10 +75,11 @@ int fa_bwd_delta(int dtype, const fa_view4* o, const fa_view4* dout, float* delt
 int fa_bwd_dkdv(int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v,
                 const fa_view4* dout, const float* lse, const float* delta, const fa_view4* dk,
                 const fa_view4* dv, int heads_per_slice, int B, int H, int Hk, int M, int N, int D,
-                int causal, float sm_scale, void* stream);
+                int causal, float sm_scale, float dropout_p, uint64_t seed, uint64_t offset, void* stream);
 int fa_bwd_dq(int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v,
               const fa_view4* dout, const float* lse, const float* delta, const fa_view4* dq, int B,
-              int H, int Hk, int M, int N, int D, int causal, float sm_scale, void* stream);
+              int H, int Hk, int M, int N, int D, int causal, float sm_scale, float dropout_p,
+              uint64_t seed, uint64_t offset, void* stream);
 
 /* The same backward with dS kept instead of recomputed (no counterpart in the reference, whose
  * `_bwd_q_kernel`, flash.py:748-909, recomputes the scores, the probabilities and dP): fa_bwd_dkdv_ds
@@ -86,7 +93,8 @@ int fa_bwd_ds_workspace_mib(int B, int H, int M, int N);
 int fa_bwd_dkdv_ds(int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v,
                    const fa_view4* dout, const float* lse, const float* delta, const fa_view4* dk,
                    const fa_view4* dv, int heads_per_slice, void* ds_workspace, int64_t ds_workspace_bytes,
-                   int B, int H, int Hk, int M, int N, int D, int causal, float sm_scale, void* stream);
+                   int B, int H, int Hk, int M, int N, int D, int causal, float sm_scale, float dropout_p,
+                   uint64_t seed, uint64_t offset, void* stream);
 int fa_bwd_dq_from_ds(int dtype, const fa_view4* k, const void* ds_workspace, int64_t ds_workspace_bytes,
                       const fa_view4* dq, int B, int H, int Hk, int M, int N, int D, int causal,
                       float sm_scale, void* stream);

@@ -22,9 +22,17 @@ randomized three-way comparison), see ``tests/test_oracle_*.py``:
 * ``paged_attention``: equals dense single-query attention on the gathered keys/values, invariant
   under a permutation of the cache blocks with the block table permuted alike; fp64 loop.
 
-No function of this oracle is "parity unpinned".
+* ``dropout.keep_mask`` (+ the ``dropout_mask`` argument of ``flash_attention``): Philox-4x32 against
+  the Random123 known-answer vectors, the uniform map against its defining properties, the drop
+  rate; dropout with an all-true mask equals no dropout; a hand-built mask against an explicit loop.
+
+No function of this oracle is "parity unpinned" with respect to what the kernels are compared
+against.  One statement is: that ``dropout.keep_mask`` reproduces, bit for bit, the mask a Triton run
+of the reference would draw -- it restates Triton's published ``tl.rand`` but no such run is possible
+here (no GPU with Triton), so bitwise mask parity with the reference is unpinned.
 """
 from .flash import flash_attention  # noqa: F401
 from .piecewise import piecewise_attention, piecewise_attention_grad  # noqa: F401
 from .paged import paged_attention  # noqa: F401
 from .compare import max_abs_diff, within_two_x  # noqa: F401
+from .dropout import keep_mask  # noqa: F401

@@ -12,7 +12,10 @@ Test infrastructure only (see the package docstring).  Follows
 * rows that see no key (``M > N`` with the causal mask) give an all ``-inf`` row, the softmax makes
   them NaN and a second select zeroes the masked probabilities (``:48-50``), so such rows produce an
   all-zero output and a log-normalizer of ``-inf``;
-* probabilities are rounded to the value dtype before the second product (``:60``).
+* probabilities are rounded to the value dtype before the second product (``:60``);
+* dropout (``:55-60``): dropped probabilities are zeroed after the normaliser, total attention and
+  log-normalizer have been taken, and the output is scaled by ``1 / (1 - dropout_p)``.  The mask is an
+  input (``oracle.dropout.keep_mask`` restates how the kernels derive it from seed and offset).
 """
 import math
 
@@ -27,7 +30,8 @@ def _visible(M, N, device):
 
 
 def flash_attention(q, k, v, causal=False, sm_scale=None, upcast=False,
-                    return_log_normalizer=False, return_total_attention=False):
+                    return_log_normalizer=False, return_total_attention=False,
+                    dropout_p=0.0, dropout_mask=None):
     """q (B, Hq, M, D); k, v (B, Hk, N, D).  Returns ``out`` or ``(out, lse|None, total|None)``.
 
     ``upcast=True`` is the fp32 reference, ``upcast=False`` the same-precision implementation that
@@ -62,7 +66,9 @@ def flash_attention(q, k, v, causal=False, sm_scale=None, upcast=False,
 
     total = probs.sum(dim=-2) if return_total_attention else None
 
-    out = torch.matmul(probs.to(v.dtype), v).to(out_dtype)
+    if dropout_mask is not None:
+        probs = probs.masked_fill(~dropout_mask, 0.0)
+    out = (torch.matmul(probs.to(v.dtype), v) * (1.0 / (1.0 - dropout_p))).to(out_dtype)
     if return_log_normalizer or return_total_attention:
         return out, lse, total
     return out

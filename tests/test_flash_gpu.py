@@ -149,8 +149,8 @@ def test_return_convention_and_asserts():
         flag_attn.flash_attention(q[..., :24], k[..., :24], v[..., :24])  # head dim not in {16,32,64,128}
     with pytest.raises(AssertionError):
         flag_attn.flash_attention(q, k[:, :1].expand(1, 3, 64, 32), v[:, :1].expand(1, 3, 64, 32))
-    with pytest.raises(NotImplementedError):
-        flag_attn.flash_attention(q, k, v, dropout_p=0.5)
+    with pytest.raises(AssertionError):
+        flag_attn.flash_attention(q, k, v, dropout_p=1.0)
 
 
 @pytest.mark.parametrize("causal", [False, True])
@@ -223,3 +223,49 @@ def test_full_size_backward_paths_agree():
     check("o", stored[0][:, hs], o_same, o_ref)
     for name, h, s, r in zip(("dq", "dk", "dv"), stored[1:], g_same, g_ref):
         check(name, h[:, hs], s, r)
+
+
+@pytest.mark.parametrize("B,Hq,Hk,M,N,D", [(2, 4, 4, 512, 612, 128), (2, 4, 2, 1024, 1034, 64), (1, 8, 2, 1300, 1300, 128),
+                                            (2, 4, 4, 777, 300, 32)])
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("dropout_p", [0.2, 0.8])
+def test_attention_dropout(B, Hq, Hk, M, N, D, causal, dtype, dropout_p):
+    """Dropout through the public API: the returned (seed, offset) reproduce the mask in the oracle's
+    restatement, and outputs and gradients then obey the 2x rule (covers the dS-kept backward at
+    head size 128 with a large score matrix, and the recomputing one)."""
+    from oracle import keep_mask
+    q = make((B, Hq, M, D), dtype, "BHTD", 1.0, 1, grad=True)
+    k = make((B, Hk, N, D), dtype, "BTHD", 1.0, 2, grad=True)
+    v = make((B, Hk, N, D), dtype, "BTHD", 1.0, 3, grad=True)
+    do = make((B, Hq, M, D), dtype, "BHTD", 1.0, 4)
+    o, L, _, seed, offset = flag_attn.flash_attention(q, k, v, causal, dropout_p=dropout_p, return_log_normalizer=True,
+                                                      return_seed_offset=True)
+    grads = torch.autograd.grad(o, (q, k, v), do)
+    assert isinstance(seed, int) and isinstance(offset, int)
+    mask = keep_mask(B, Hq, M, N, dropout_p, seed, offset, device="cuda")
+    assert abs((~mask).float().mean().item() - dropout_p) < 0.01
+    ref = oracle_flash(q, k, v, causal, upcast=True, return_log_normalizer=True, dropout_p=dropout_p, dropout_mask=mask)
+    same = oracle_flash(q, k, v, causal, upcast=False, return_log_normalizer=True, dropout_p=dropout_p, dropout_mask=mask)
+    g_ref = torch.autograd.grad(ref[0], (q, k, v), do)
+    g_same = torch.autograd.grad(same[0], (q, k, v), do)
+    check("o", o, same[0], ref[0])
+    check("L", L, same[1], ref[1])
+    for name, h, s, r in zip(("dq", "dk", "dv"), grads, g_same, g_ref):
+        check(name, h, s, r)
+
+
+def test_dropout_advances_the_generator_and_is_reproducible():
+    q, k, v = (make((2, 16, 256, 64), torch.float16, "BHTD", 1.0, s) for s in (1, 2, 3))
+    torch.cuda.manual_seed(4321)
+    o1, _, _, s1, off1 = flag_attn.flash_attention(q, k, v, dropout_p=0.5, return_seed_offset=True)
+    o2, _, _, s2, off2 = flag_attn.flash_attention(q, k, v, dropout_p=0.5, return_seed_offset=True)
+    assert s1 == s2 == 4321 and off2 == off1 + 2 * 16 * 256 * 256      # offset advanced by B * H * M * N
+    assert not torch.equal(o1, o2)
+    torch.cuda.manual_seed(4321)
+    o3 = flag_attn.flash_attention(q, k, v, dropout_p=0.5)
+    assert torch.equal(o1, o3)
+    assert flag_attn.flash_attention(q, k, v, dropout_p=0.0, return_seed_offset=True)[3:] == (None, None)
+    with pytest.raises(AssertionError):   # decode shapes take the split-KV path, which has no dropout
+        flag_attn.flash_attention(q[:1, :2, :1], make((1, 2, 8192, 64), torch.float16, "BHTD", 1.0, 5),
+                                  make((1, 2, 8192, 64), torch.float16, "BHTD", 1.0, 6), dropout_p=0.5)

@@ -130,6 +130,63 @@ def test_flash_backward_with_stored_ds(lib, B, H, Hk, M, N, D, causal, dtype, bt
     assert (dq.float() - dq_plain.float()).abs().max() <= 2e-2 * dq_plain.float().abs().max() + 1e-6
 
 
+DROPOUT_CASES = [
+    # B, H, Hk, M, N, D, causal, dtype, p, seed, offset
+    (1, 2, 1, 70, 100, 64, True, torch.bfloat16, 0.3, 1234, 40),
+    (2, 1, 1, 40, 40, 128, False, torch.float16, 0.5, 987654321987, 123456789123456789),   # 64-bit counter
+    (1, 2, 2, 130, 70, 32, True, torch.float16, 0.1, 7, 0),                               # rows without keys
+]
+
+
+@pytest.mark.parametrize("B,H,Hk,M,N,D,causal,dtype,pd,seed,offset", DROPOUT_CASES)
+def test_flash_dropout(lib, B, H, Hk, M, N, D, causal, dtype, pd, seed, offset):
+    """Forward, both backward routes (dS recomputed / dS kept) with dropout, against the oracle given
+    the mask that oracle.dropout restates from (seed, offset)."""
+    from oracle import keep_mask
+    q = rnd((B, H, M, D), dtype).requires_grad_()
+    k = rnd((B, Hk, N, D), dtype).requires_grad_()
+    v = rnd((B, Hk, N, D), dtype).requires_grad_()
+    do = rnd((B, H, M, D), dtype)
+    sc = 1 / math.sqrt(D)
+    drop = (pd, seed, offset)
+    qd, kd, vd = q.detach(), k.detach(), v.detach()
+    o = torch.full_like(qd, float("nan"))
+    lse = torch.full((B, H, M), float("nan"))
+    _abi.fa_fwd(lib, qd, kd, vd, o, lse, causal, sc, drop)
+    delta = torch.full((B, H, M), float("nan"))
+    _abi.fa_bwd_delta(lib, o, do, delta)
+    # with dropout the kernels leave one dK/dV slice per query head
+    dk, dv = torch.empty(B, H, N, D, dtype=dtype), torch.empty(B, H, N, D, dtype=dtype)
+    dq = torch.empty(B, H, M, D, dtype=dtype)
+    if H > Hk:
+        with pytest.raises(AssertionError):
+            _abi.fa_bwd_dkdv(lib, qd, kd, vd, do, lse, delta, dk[:, :Hk], dv[:, :Hk], causal, sc, drop)
+    _abi.fa_bwd_dkdv(lib, qd, kd, vd, do, lse, delta, dk, dv, causal, sc, drop)
+    _abi.fa_bwd_dq(lib, qd, kd, vd, do, lse, delta, dq, causal, sc, drop)
+    dk2, dv2, dq2 = torch.empty_like(dk), torch.empty_like(dv), torch.empty_like(dq)
+    ds = torch.full((lib.fa_bwd_ds_workspace_mib(B, H, M, N) << 19,), float("nan"), dtype=dtype)
+    _abi.fa_bwd_dkdv_ds(lib, qd, kd, vd, do, lse, delta, dk2, dv2, ds, causal, sc, drop)
+    _abi.fa_bwd_dq_from_ds(lib, kd, ds, dq2, causal, sc)
+    assert torch.equal(dk, dk2) and torch.equal(dv, dv2)
+    dk, dv = dk.reshape(B, Hk, H // Hk, N, D).sum(2), dv.reshape(B, Hk, H // Hk, N, D).sum(2)
+
+    mask = keep_mask(B, H, M, N, pd, seed, offset)
+    assert 0 < (~mask).float().mean() < 1
+    ref = flash_attention(q, k, v, causal, upcast=True, return_log_normalizer=True, dropout_p=pd, dropout_mask=mask)
+    same = flash_attention(q, k, v, causal, upcast=False, return_log_normalizer=True, dropout_p=pd, dropout_mask=mask)
+    g_ref = torch.autograd.grad(ref[0], (q, k, v), do)
+    g_same = torch.autograd.grad(same[0], (q, k, v), do)
+    check("o", o, same[0], ref[0])
+    check("lse", lse, same[1], ref[1])
+    for name, h, s_, r in (("dq", dq, g_same[0], g_ref[0]), ("dq (dS kept)", dq2, g_same[0], g_ref[0]),
+                           ("dk", dk, g_same[1], g_ref[1]), ("dv", dv, g_same[2], g_ref[2])):
+        check(name, h, s_, r)
+    # a different seed gives a different output: the mask is really applied
+    o2 = torch.empty_like(o)
+    _abi.fa_fwd(lib, qd, kd, vd, o2, lse, causal, sc, (pd, seed + 1, offset))
+    assert not torch.equal(o, o2)
+
+
 PW_CASES = [
     # B, H, M, N, D, w, causal, dtype
     (1, 2, 200, 200, 64, 50, True, torch.bfloat16),
