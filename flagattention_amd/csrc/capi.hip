@@ -267,7 +267,7 @@ int paged_attn(int dtype, void* out, int64_t o_stride_s, int64_t o_stride_h, con
   if (!query || !key_cache || !value_cache || !block_tables) return FA_ERR_BAD_ARGUMENT;
   if ((((uintptr_t)query) | ((uintptr_t)key_cache) | ((uintptr_t)value_cache)) & 15) return FA_ERR_BAD_ARGUMENT;
   if ((q_stride_s | q_stride_h | kv_stride_blk | kv_stride_h | kv_stride_tok) % 8) return FA_ERR_BAD_ARGUMENT;
-  if (!(head_size == 16 || head_size == 32 || head_size == 64 || head_size == 128 || head_size == 256))
+  if (!(head_size == 16 || head_size == 32 || head_size == 64 || head_size == 128 || head_size == 256 || head_size == 512))
     return FA_ERR_UNSUPPORTED;
   p.q = query; p.q_ss = q_stride_s; p.q_sh = q_stride_h;
   p.kc = key_cache; p.vc = value_cache;
@@ -298,7 +298,7 @@ int paged_attn_balanced(int dtype, void* out, int64_t o_stride_s, int64_t o_stri
   if ((((uintptr_t)query) | ((uintptr_t)key_cache) | ((uintptr_t)value_cache) | ((uintptr_t)workspace)) & 15)
     return FA_ERR_BAD_ARGUMENT;
   if ((q_stride_s | q_stride_h | kv_stride_blk | kv_stride_h | kv_stride_tok) % 8) return FA_ERR_BAD_ARGUMENT;
-  if (!(head_size == 16 || head_size == 32 || head_size == 64 || head_size == 128 || head_size == 256))
+  if (!(head_size == 16 || head_size == 32 || head_size == 64 || head_size == 128 || head_size == 256 || head_size == 512))
     return FA_ERR_UNSUPPORTED;
   if (num_workgroups <= 0 || workspace_bytes < fa::paged_balanced_workspace_bytes(num_workgroups, head_size))
     return FA_ERR_BAD_ARGUMENT;

@@ -27,7 +27,11 @@ namespace fa {
 
 template <class T, int D>
 struct DecCfg {
-  static constexpr int TK = 32;    // keys per wavefront step
+  // keys per wavefront step: two 16-key score blocks fill the contraction of the second product; at
+  // head size 512 a 32-key step would not fit registers (loads in flight) or LDS (4 patches), so the
+  // step is one block and the other half of the contraction multiplies zeros (the kernel is HBM-bound)
+  static constexpr int TK = D > 256 ? 16 : 32;
+  static constexpr int KB = TK / 16;  // 16-key score blocks per step
   static constexpr int ROWS = 16;  // query rows per workgroup
   static constexpr int DK = D < 32 ? 32 : D;  // contraction width of the first product (zero padded)
   static constexpr int KSTEPS = DK / 32;
@@ -41,7 +45,11 @@ struct DecCfg {
   static constexpr size_t STAGING_BYTES = 4 * WAVE_ELEMS * sizeof(T);
   // merge area: per wavefront ROWS x (D + 2) floats
   static constexpr size_t MERGE_BYTES = 4 * ROWS * (D + 2) * sizeof(float);
-  static constexpr size_t LDS_BYTES = STAGING_BYTES > MERGE_BYTES ? STAGING_BYTES : MERGE_BYTES;
+  static constexpr size_t WORK_BYTES = STAGING_BYTES > MERGE_BYTES ? STAGING_BYTES : MERGE_BYTES;
+  // at head size 512 the query rows (64 registers as an MFMA operand) live in LDS behind the work area
+  static constexpr bool Q_IN_LDS = D > 256;
+  static constexpr int Q_LD = DK + 8;
+  static constexpr size_t LDS_BYTES = WORK_BYTES + (Q_IN_LDS ? ROWS * Q_LD * sizeof(T) : 0);
 };
 
 // Result of the per-workgroup pass, valid in every thread after decode_block():
@@ -71,12 +79,22 @@ FA_DEVICE void decode_block(const Src& src, const T* q_row /* query row of lane 
   T* sV = sK + C::TK * C::K_LD;
 
   // this lane's query row as B operand: contraction indices 32 ks + 8 g + 0..7
-  V8 qreg[C::KSTEPS];
+  V8 qreg[C::Q_IN_LDS ? 1 : C::KSTEPS];
+  T* sQ = (T*)(smem + C::WORK_BYTES);
+  if (C::Q_IN_LDS) {  // wavefront w stores every fourth 32-wide slice of the 16 rows
+    for (int ks = wave; ks < C::KSTEPS; ks += 4) {
+      u32x4 z = {0u, 0u, 0u, 0u};
+      if (q_row) z = *(const u32x4*)(q_row + 32 * ks + 8 * g);
+      *(u32x4*)(sQ + li * C::Q_LD + 32 * ks + 8 * g) = z;
+    }
+    hw::block_sync();
+  } else {
 #pragma unroll
-  for (int ks = 0; ks < C::KSTEPS; ++ks) {
-    u32x4 z = {0u, 0u, 0u, 0u};
-    if (q_row && 32 * ks + 8 * g < D) z = *(const u32x4*)(q_row + 32 * ks + 8 * g);
-    qreg[ks] = hw::as_v8<T>(z);
+    for (int ks = 0; ks < C::KSTEPS; ++ks) {
+      u32x4 z = {0u, 0u, 0u, 0u};
+      if (q_row && 32 * ks + 8 * g < D) z = *(const u32x4*)(q_row + 32 * ks + 8 * g);
+      qreg[ks] = hw::as_v8<T>(z);
+    }
   }
   if (C::DK != D) {  // columns D..DK-1 of the key patch are read by the first product, never loaded
     for (int i = lane; i < C::TK * C::K_LD; i += 64) sK[i] = (T)0.f;
@@ -140,27 +158,35 @@ FA_DEVICE void decode_block(const Src& src, const T* q_row /* query row of lane 
     }
     hw::wave_sync();
 
-    // ---- S^T: two blocks of 16 keys x 16 queries ----
-    hw::f32x4 s[2];
-    {
-      V8 ka[2][C::KSTEPS];  // all operands requested before the first product: one exposed LDS latency
+    // ---- S^T: blocks of 16 keys x 16 queries ----
+    hw::f32x4 s[C::KB];
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
+    for (int kb = 0; kb < C::KB; ++kb) s[kb] = hw::f32x4{0.f, 0.f, 0.f, 0.f};
+    constexpr int kKGroup = C::KSTEPS < 8 ? C::KSTEPS : 8;
 #pragma unroll
-        for (int ks = 0; ks < C::KSTEPS; ++ks)
-          ka[kb][ks] = hw::as_v8<T>(*(const u32x4*)(sK + (16 * kb + li) * C::K_LD + 32 * ks + 8 * g));
+    for (int k0 = 0; k0 < C::KSTEPS; k0 += kKGroup) {
+      V8 ka[C::KB][kKGroup];  // operands requested before the first product of the group: one exposed LDS latency
+      V8 qb[kKGroup];
+#pragma unroll
+      for (int ks = 0; ks < kKGroup; ++ks)
+      {
+        if constexpr (C::Q_IN_LDS) qb[ks] = hw::as_v8<T>(*(const u32x4*)(sQ + li * C::Q_LD + 32 * (k0 + ks) + 8 * g));
+        else qb[ks] = qreg[k0 + ks];
+      }
+#pragma unroll
+      for (int kb = 0; kb < C::KB; ++kb)
+#pragma unroll
+        for (int ks = 0; ks < kKGroup; ++ks)
+          ka[kb][ks] = hw::as_v8<T>(*(const u32x4*)(sK + (16 * kb + li) * C::K_LD + 32 * (k0 + ks) + 8 * g));
       hw::sched_fence();
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
-        hw::f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+      for (int kb = 0; kb < C::KB; ++kb)
 #pragma unroll
-        for (int ks = 0; ks < C::KSTEPS; ++ks) acc = hw::mfma16(ka[kb][ks], qreg[ks], acc);
-        s[kb] = acc;
-      }
+        for (int ks = 0; ks < kKGroup; ++ks) s[kb] = hw::mfma16(ka[kb][ks], qb[ks], s[kb]);
     }
     float mx = neg_inf();
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
+    for (int kb = 0; kb < C::KB; ++kb)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int n = n0 + 16 * kb + 4 * g + r;
@@ -178,7 +204,9 @@ FA_DEVICE void decode_block(const Src& src, const T* q_row /* query row of lane 
     float psum = 0.f;
     V8 pb;
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
+    for (int i = 0; i < 8; ++i) pb[i] = (T)0.f;
+#pragma unroll
+    for (int kb = 0; kb < C::KB; ++kb)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const float e = hw::exp2_fast(fmaf(s[kb][r], c2, shift));
@@ -195,7 +223,8 @@ FA_DEVICE void decode_block(const Src& src, const T* q_row /* query row of lane 
 #pragma unroll
       for (int u = 0; u < kGroup; ++u) {
         const T* pv = sV + (4 * g + (li >> 2)) * C::V_LD + 16 * (d0 + u) + 4 * (li & 3);
-        va[u] = hw::join_v8<T>(hw::lds_read_tr16(pv), hw::lds_read_tr16(pv + 16 * C::V_LD));
+        const hw::short4v lo = hw::lds_read_tr16(pv);
+        va[u] = hw::join_v8<T>(lo, C::KB == 2 ? hw::lds_read_tr16(pv + (C::KB - 1) * 16 * C::V_LD) : hw::short4v{0, 0, 0, 0});
       }
       hw::sched_fence();
 #pragma unroll

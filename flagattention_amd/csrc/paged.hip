@@ -216,7 +216,9 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (D <= 128 ? 2 : 1)) paged_balanced_ke
     hw::block_sync();
     int* t = scan_a; scan_a = scan_b; scan_b = t;
   }
-  const int64_t total = (int64_t)scan_a[kThreads - 1] * pairs_per_seq;
+  // read through a scalar register: everything derived from it (the key ranges, the step counts of
+  // the wavefronts) then stays in scalar registers too
+  const int64_t total = (int64_t)hw::uniform(scan_a[kThreads - 1]) * pairs_per_seq;
   const int64_t per = (int64_t)imax(kMinUnitsPerWg, (int)((total + p.num_wgs - 1) / p.num_wgs));
   const int64_t u_begin = (int64_t)w * per;
   const int64_t u_end = u_begin + per < total ? u_begin + per : total;
@@ -331,6 +333,7 @@ static int launch_balanced(const PagedParams& p, hipStream_t stream) {
     case 64: return launch_balanced_d<T, 64>(p, stream);
     case 128: return launch_balanced_d<T, 128>(p, stream);
     case 256: return launch_balanced_d<T, 256>(p, stream);
+    case 512: return launch_balanced_d<T, 512>(p, stream);
   }
   return kUnsupported;
 }
@@ -346,6 +349,7 @@ static int launch_paged(const PagedParams& p, hipStream_t stream) {
     case 64: return launch(paged_attn_kernel<T, 64>, grid, DecCfg<T, 64>::LDS_BYTES, stream, p);
     case 128: return launch(paged_attn_kernel<T, 128>, grid, DecCfg<T, 128>::LDS_BYTES, stream, p);
     case 256: return launch(paged_attn_kernel<T, 256>, grid, DecCfg<T, 256>::LDS_BYTES, stream, p);
+    case 512: return launch(paged_attn_kernel<T, 512>, grid, DecCfg<T, 512>::LDS_BYTES, stream, p);
   }
   return kUnsupported;
 }

@@ -10,7 +10,7 @@ from . import _abi, _lib
 
 __all__ = ["attention"]
 
-_HEAD_SIZES = (16, 32, 64, 128, 256)
+_HEAD_SIZES = (16, 32, 64, 128, 256, 512)
 
 
 def _next_pow2(x):
@@ -22,7 +22,7 @@ def choose_launch(num_seqs, num_kv_heads, group, head_size, max_context_len, num
 
     Returns ("balanced", num_workgroups) or ("single", 0).  The balanced launch divides the keys of
     all (sequence, kv head) pairs evenly over one resident wave of workgroups (two per compute unit
-    fit up to head size 128, one at 256) and so does not depend on how the context lengths are
+    fit up to head size 128, one above) and so does not depend on how the context lengths are
     spread; its fixed cost (a scan of the context lengths per workgroup, a merge kernel) only loses
     against one workgroup per pair when there are many more short pairs than workgroups, where the
     hardware's own dispatch already evens things out."""

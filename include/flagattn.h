@@ -146,6 +146,7 @@ int pw_bwd_dq(int dtype, const fa_view4* q1, const fa_view4* k1, const fa_view4*
  * query (num_seqs, Hq, D) with element strides q_stride_s, q_stride_h; key_cache / value_cache
  * (num_blocks, Hkv, block_size, D) sharing the element strides kv_stride_{blk,h,tok};
  * context_lens int32; block_tables int32 or int64 (bt_is_int64) with row stride bt_stride.
+ * head_size in {16, 32, 64, 128, 256, 512} (paged.py:31).
  * partition_size == 0: one pass, `out` (num_seqs, Hq, D) with strides o_stride_s, o_stride_h.
  * partition_size > 0 (a multiple of block_size): grid over num_parts partitions; writes
  * tmp_out (num_seqs, Hkv, num_parts, G, D) in the cache dtype and max_logits / exp_sums
@@ -167,7 +168,7 @@ int paged_reduce(int dtype, void* out, int64_t o_stride_s, int64_t o_stride_h, c
  * `num_splits == 0` branch) together with the two launches it leads to (:57-162).  Instead of
  * cutting every sequence into partitions of one size, the keys of all (sequence, kv head) pairs are
  * laid end to end and divided evenly over num_workgroups workgroups (use twice the number of compute
- * units for head_size <= 128, once for 256); pairs cut by a boundary are merged by a second kernel
+ * units for head_size <= 128, once above); pairs cut by a boundary are merged by a second kernel
  * launched by the same call.  `workspace` is device memory of at least
  * paged_attn_balanced_workspace(num_workgroups, head_size) bytes, 16-byte aligned; its contents on
  * entry do not matter and it may be reused by the next call on the same stream. */

@@ -70,10 +70,17 @@ def test_paged_attention_by_case(num_seqs, num_query_heads, query_group_size, he
     run_case(num_seqs, num_query_heads, query_group_size, head_size, block_size, max_seq_len, num_splits)
 
 
-@pytest.mark.parametrize("head_size", [16, 256])
+@pytest.mark.parametrize("head_size", [16, 256, 512])
 @pytest.mark.parametrize("table_dtype", [torch.int32, torch.int64])
 def test_other_head_sizes_and_table_types(head_size, table_dtype):
     run_case(4, 16, 4, head_size, 32, 700, table_dtype=table_dtype)
+
+
+@pytest.mark.parametrize("num_splits", [0, 1, 3])
+def test_head_size_512(num_splits):
+    """The largest head size of the reference (paged.py:31): the kernel walks 16-key steps there."""
+    run_case(6, 8, 2, 512, 16, 1500, num_splits=num_splits)
+    run_case(3, 4, 1, 512, 16, 333, num_splits=num_splits, dtype=torch.bfloat16)
 
 
 def test_bfloat16_and_large_group():

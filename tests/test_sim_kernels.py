@@ -259,6 +259,9 @@ PAGED_CASES = [
     (2, 4, 1, 64, 16, 2, 1, 0, torch.float16, torch.int64),
     (2, 6, 2, 16, 32, 200, 2, 128, torch.bfloat16, torch.int64),
     (1, 40, 40, 64, 16, 70, 2, 64, torch.float16, torch.int64),
+    (2, 4, 2, 256, 16, 150, 1, 0, torch.float16, torch.int64),
+    (2, 4, 2, 512, 16, 150, 1, 0, torch.float16, torch.int64),   # 16-key steps
+    (2, 2, 1, 512, 16, 200, 2, 128, torch.bfloat16, torch.int32),
 ]
 
 
@@ -296,6 +299,7 @@ BALANCED_CASES = [
     (2, 40, 40, 32, 8, [200, 90], 4, torch.bfloat16, torch.int64),          # 3 row blocks per kv head
     (5, 2, 2, 16, 16, [40, 50, 60, 70, 80], 64, torch.float16, torch.int64),  # more workgroups than work
     (1, 2, 1, 64, 16, [1500], 5, torch.float16, torch.int64),               # one pair over many workgroups
+    (2, 4, 4, 512, 16, [300, 77], 3, torch.float16, torch.int64),           # 16-key steps
 ]
 
 
