@@ -154,6 +154,23 @@ def pw_bwd_dq(lib, q1, k1, q2, k2, v, do, lse, delta, dq1, dq2, w, causal, sm_sc
                         int(causal), float(sm_scale), stream_of(q1)), "pw_bwd_dq")
 
 
+def pw_bwd_dkdv_ds(lib, q1, k1, q2, k2, v, do, lse, delta, dk1, dk2, dv, ds, w, causal, sm_scale):
+    B, H, M, D = q1.shape
+    N = k1.shape[2]
+    check(lib.pw_bwd_dkdv_ds(dtype_code(q1), view4(q1), view4(k1), view4(q2), view4(k2), view4(v), view4(do),
+                             ptr(lse), ptr(delta), view4(dk1), view4(dk2), view4(dv), ptr(ds),
+                             ds.numel() * ds.element_size(), B, H, M, N, D, int(w), int(causal),
+                             float(sm_scale), stream_of(q1)), "pw_bwd_dkdv_ds")
+
+
+def pw_bwd_dq_from_ds(lib, k1, k2, ds, dq1, dq2, w, causal, sm_scale):
+    B, H, M, D = dq1.shape
+    N = k1.shape[2]
+    check(lib.pw_bwd_dq_from_ds(dtype_code(dq1), view4(k1), view4(k2), ptr(ds), ds.numel() * ds.element_size(),
+                                view4(dq1), view4(dq2), B, H, M, N, D, int(w), int(causal),
+                                float(sm_scale), stream_of(dq1)), "pw_bwd_dq_from_ds")
+
+
 def fa_total_attn(lib, q, k, lse, total, causal, sm_scale):
     B, H, M, D = q.shape
     Hk, N = k.shape[1], k.shape[2]

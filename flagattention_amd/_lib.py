@@ -37,6 +37,8 @@ SIGNATURES = {
     "pw_fwd": [_i, _v, _v, _v, _v, _v, _v, _p, _i, _i, _i, _i, _i, _i, _i, _f, _p],
     "pw_bwd_dkdv": [_i, _v, _v, _v, _v, _v, _v, _p, _p, _v, _v, _v, _i, _i, _i, _i, _i, _i, _i, _f, _p],
     "pw_bwd_dq": [_i, _v, _v, _v, _v, _v, _v, _p, _p, _v, _v, _i, _i, _i, _i, _i, _i, _i, _f, _p],
+    "pw_bwd_dkdv_ds": [_i, _v, _v, _v, _v, _v, _v, _p, _p, _v, _v, _v, _p, _i64, _i, _i, _i, _i, _i, _i, _i, _f, _p],
+    "pw_bwd_dq_from_ds": [_i, _v, _v, _p, _i64, _v, _v, _i, _i, _i, _i, _i, _i, _i, _f, _p],
     "paged_attn": [_i, _p, _i64, _i64, _p, _i64, _i64, _p, _p, _i64, _i64, _i64, _p, _p, _i, _i64, _f,
                    _i, _i, _i, _i, _i, _i, _i, _p, _p, _p, _p],
     "paged_reduce": [_i, _p, _i64, _i64, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p],

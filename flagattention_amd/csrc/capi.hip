@@ -147,7 +147,7 @@ int fa_bwd_dkdv_ds(int dtype, const fa_view4* q, const fa_view4* k, const fa_vie
   p.chunk = heads_per_slice;
   p.dropout_p = dropout_p; p.seed = seed; p.offset = offset;
   p.ds = ds_workspace;
-  return fa::run_bwd_dkdv_ds(p, (hipStream_t)stream);
+  return fa::run_bwd_dkdv_ds(p, false, (hipStream_t)stream);
 }
 
 int fa_bwd_dq_from_ds(int dtype, const fa_view4* k, const void* ds_workspace, int64_t ds_workspace_bytes,
@@ -164,7 +164,7 @@ int fa_bwd_dq_from_ds(int dtype, const fa_view4* k, const void* ds_workspace, in
   p.ds = const_cast<void*>(ds_workspace);
   p.B = B; p.H = H; p.M = M; p.N = N; p.D = D; p.group = H / Hk;
   p.causal = causal; p.sm_scale = sm_scale; p.dtype = dtype;
-  return fa::run_bwd_dq_from_ds(p, (hipStream_t)stream);
+  return fa::run_bwd_dq_from_ds(p, false, (hipStream_t)stream);
 }
 
 int pw_bwd_dkdv(int dtype, const fa_view4* q1, const fa_view4* k1, const fa_view4* q2,
@@ -195,6 +195,46 @@ int pw_bwd_dq(int dtype, const fa_view4* q1, const fa_view4* k1, const fa_view4*
   p.dq = to_view(dq1); p.dq2 = to_view(dq2);
   p.w = dist_threshold;
   return fa::run_bwd_dq(p, true, (hipStream_t)stream);
+}
+
+int pw_bwd_dkdv_ds(int dtype, const fa_view4* q1, const fa_view4* k1, const fa_view4* q2,
+                   const fa_view4* k2, const fa_view4* v, const fa_view4* dout, const float* lse,
+                   const float* delta, const fa_view4* dk1, const fa_view4* dk2, const fa_view4* dv,
+                   void* ds_workspace, int64_t ds_workspace_bytes, int B, int H, int M, int N, int D,
+                   int dist_threshold, int causal, float sm_scale, void* stream) {
+  fa::BwdParams p = {};
+  int rc = fill_bwd(p, dtype, q1, k1, v, dout, lse, delta, B, H, H, M, N, D, causal, sm_scale);
+  if (rc) return rc;
+  if (!view_ok(q2) || !view_ok(k2) || !view_ok(dk1) || !view_ok(dk2) || !view_ok(dv))
+    return FA_ERR_BAD_ARGUMENT;
+  if (!ds_workspace || (((uintptr_t)ds_workspace) & 15) ||
+      ds_workspace_bytes < 2 * fa::bwd_ds_workspace_bytes(B, H, M, N))
+    return FA_ERR_BAD_ARGUMENT;
+  p.q2 = to_view(q2); p.k2 = to_view(k2);
+  p.dk = to_view(dk1); p.dk2 = to_view(dk2); p.dv = to_view(dv);
+  p.w = dist_threshold;
+  p.ds = ds_workspace;
+  return fa::run_bwd_dkdv_ds(p, true, (hipStream_t)stream);
+}
+
+int pw_bwd_dq_from_ds(int dtype, const fa_view4* k1, const fa_view4* k2, const void* ds_workspace,
+                      int64_t ds_workspace_bytes, const fa_view4* dq1, const fa_view4* dq2, int B, int H,
+                      int M, int N, int D, int dist_threshold, int causal, float sm_scale, void* stream) {
+  if (!view_ok(k1) || !view_ok(k2) || !view_ok(dq1) || !view_ok(dq2)) return FA_ERR_BAD_ARGUMENT;
+  if (!head_dim_ok(D)) return FA_ERR_UNSUPPORTED;
+  if (B <= 0 || H <= 0 || M <= 0 || N <= 0) return FA_ERR_BAD_ARGUMENT;
+  if (!ds_workspace || (((uintptr_t)ds_workspace) & 15) ||
+      ds_workspace_bytes < 2 * fa::bwd_ds_workspace_bytes(B, H, M, N))
+    return FA_ERR_BAD_ARGUMENT;
+  fa::BwdParams p = {};
+  p.ds = const_cast<void*>(ds_workspace);
+  p.B = B; p.H = H; p.M = M; p.N = N; p.D = D; p.group = 1;
+  p.causal = causal; p.w = dist_threshold; p.sm_scale = sm_scale; p.dtype = dtype;
+  p.k = to_view(k1); p.dq = to_view(dq1); p.regime = 1;
+  int rc = fa::run_bwd_dq_from_ds(p, true, (hipStream_t)stream);
+  if (rc) return rc;
+  p.k = to_view(k2); p.dq = to_view(dq2); p.regime = 2;
+  return fa::run_bwd_dq_from_ds(p, true, (hipStream_t)stream);
 }
 
 int fa_total_attn(int dtype, const fa_view4* q, const fa_view4* k, const float* lse, float* total,

@@ -99,7 +99,6 @@ struct KvCfg {
 template <class T, int D, bool PW, bool DS = false, bool DROP = false, bool GROUPED = false>
 FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PER_SIMD)) fa_bwd_dkdv_kernel(BwdParams p) {
   static_assert(!(GROUPED && (PW || DROP)), "grouped accumulation is built for plain attention without dropout");
-  static_assert(!(PW && DS), "the dS workspace is only defined for plain flash attention");
   static_assert(!(PW && DROP), "piecewise attention has no dropout");
   using C = KvCfg<T, D, PW>;
   using V8 = typename hw::Elem<T>::v8;
@@ -213,14 +212,19 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
   gb = (const T*)p.dout.ptr + batch * p.dout.sb + head * p.dout.sh;
   lse = p.lse + ((int64_t)batch * p.H + head) * M;
   dlt = p.delta + ((int64_t)batch * p.H + head) * M;
+  T* ds_near = nullptr;
+  int64_t ds_regime_stride = 0;  // piecewise: the far regime's chunk grid follows the near regime's
   if (DS) {
     const int64_t nqb = 4 * (int64_t)cdiv(M, 128), nkb = 4 * (int64_t)cdiv(N, 128);
-    ds_row = (T*)p.ds + ((((int64_t)batch * p.H + head) * nkb + (n0 / 32 + wave)) * nqb) * 1024 + lane * 8;
+    ds_near = (T*)p.ds + ((((int64_t)batch * p.H + head) * nkb + (n0 / 32 + wave)) * nqb) * 1024 + lane * 8;
+    ds_regime_stride = (int64_t)p.B * p.H * nkb * nqb * 1024;
+    ds_row = ds_near;
   }
   if (DROP) drop_col = p.offset + ((uint64_t)batch * p.H + head) * M * (uint64_t)N + (uint64_t)(my_n < N ? my_n : 0);
 #pragma unroll
   for (int ph = 0; ph < (PW ? 2 : 1); ++ph) {
     far_phase = PW && ph == 1;
+    if (DS && PW) ds_row = ds_near + (far_phase ? ds_regime_stride : 0);
     // query tiles [t_begin, t_end) of 64 rows that hold an entry of this regime for some key of the block
     int t_begin = m_lo / C::BM, t_end = cdiv(M, C::BM);
     if (PW) {
@@ -575,7 +579,7 @@ struct QdsCfg {
   static constexpr size_t LDS_BYTES = 2 * STAGE_BYTES;
 };
 
-template <class T, int D>
+template <class T, int D, bool PW = false>
 FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, 2) fa_bwd_dq_from_ds_kernel(BwdParams p) {
   using C = QdsCfg<T, D>;
   using V8 = typename hw::Elem<T>::v8;
@@ -595,11 +599,19 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, 2) fa_bwd_dq_from_ds_kernel(BwdParams
   const T* kb = (const T*)p.k.ptr + batch * p.k.sb + hk * p.k.sh;
   const int64_t nqb = 4 * (int64_t)cdiv(M, 128), nkb = 4 * (int64_t)cdiv(N, 128);
   // chunk (key block 0, this wavefront's query block); a key block further is nqb chunks further
+  const bool far = PW && p.regime == 2;
   const T* ds_col = (const T*)p.ds + ((((int64_t)batch * p.H + head) * nkb) * nqb + mw / 32) * 1024 + lane * 8;
+  if (far) ds_col += (int64_t)p.B * p.H * nkb * nqb * 1024;
 
-  int hi = N;
+  // key tiles that hold an entry of this launch's regime for some row of the block
+  int lo = 0, hi = N;
   if (p.causal) hi = imin(N, pseq + m0 + C::BM);
-  const int n_tiles = hi > 0 ? cdiv(hi, C::BN) : 0;
+  if (PW) {
+    if (far) hi = imin(hi, m0 + C::BM - 1 + pseq - p.w + 1);  // far: n <= m + pseq - w
+    else lo = imax(0, m0 + pseq - p.w + 1);                    // near: n > m + pseq - w
+  }
+  const int t_lo = lo / C::BN;
+  const int n_tiles = hi > lo ? cdiv(hi, C::BN) : t_lo;
 
   if (C::DV != D) {
     for (int i = tid; i < (int)(C::LDS_BYTES / sizeof(T)); i += kThreads) lds[i] = (T)0.f;
@@ -613,7 +625,12 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, 2) fa_bwd_dq_from_ds_kernel(BwdParams
     for (int r = 0; r < 16; ++r) dq[i][r] = 0.f;
 
   // a 32-key block contributes unless the mask hides all of it from this wavefront's rows
-  auto block_used = [&](int nlo) { return live && !(p.causal && (mw + 31 + pseq < nlo)); };
+  // (the same conditions under which the dK/dV kernel computed, and stored, the block)
+  auto block_used = [&](int nlo) {
+    bool used = live && !(p.causal && (mw + 31 + pseq < nlo));
+    if (PW) used = used && !(far ? (mw + 31 + pseq - nlo < p.w) : (mw + pseq - (nlo + 31) >= p.w));
+    return used;
+  };
 
   TileMover<T, C::BN, D> kr;
   kr.init(tid, p.k.st);
@@ -646,15 +663,16 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, 2) fa_bwd_dq_from_ds_kernel(BwdParams
   const int G = lane >> 4, r = lane & 15, e4 = r >> 2, a = r & 3;
   const int tr_off = (G & 1) * C::VEC + (a & 1) * (256 + 32) + (4 * (G >> 1) + e4) * 8 + 4 * (a >> 1);
 
-  if (n_tiles > 0) { fetch(0); commit(0); }
+  if (n_tiles > t_lo) { fetch(t_lo * C::BN); commit(0); }
   hw::block_sync();
 
-  for (int it = 0; it < n_tiles; ++it) {
+  int stage = 0;
+  for (int it = t_lo; it < n_tiles; ++it) {
     const int n0 = it * C::BN;
     const bool more = it + 1 < n_tiles;
     if (more) fetch(n0 + C::BN);
 
-    const T* sK = (const T*)(smem + (it & 1) * C::STAGE_BYTES);
+    const T* sK = (const T*)(smem + stage * C::STAGE_BYTES);
     const T* patch = sK + C::TILE + wave * C::PATCH;
 #pragma unroll
     for (int nb = 0; nb < 2; ++nb) {
@@ -669,8 +687,9 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, 2) fa_bwd_dq_from_ds_kernel(BwdParams
       }
     }
 
-    if (more) commit((it + 1) & 1);
+    if (more) commit(stage ^ 1);
     hw::block_sync();
+    stage ^= 1;
   }
 
   if (my_m < M) {
@@ -731,7 +750,7 @@ static bool dkdv_chunk_ok(const BwdParams& p, bool piecewise) {
 
 template <class T>
 static int dispatch_dkdv(const BwdParams& p, bool piecewise, bool keep_ds, hipStream_t stream) {
-  if (piecewise) return launch_dkdv<T, true, false, false, false>(p, stream);
+  if (piecewise) return keep_ds ? launch_dkdv<T, true, true, false, false>(p, stream) : launch_dkdv<T, true, false, false, false>(p, stream);
   const bool drop = p.dropout_p > 0.f;
   const bool grouped = (p.chunk > 0 ? p.chunk : p.group) > 1;
   if (keep_ds) {
@@ -762,14 +781,14 @@ int run_bwd_dq(const BwdParams& p, bool piecewise, hipStream_t stream) {
   return kUnsupported;
 }
 
-template <class T>
+template <class T, bool PW>
 static int launch_dq_from_ds(const BwdParams& p, hipStream_t stream) {
   dim3 grid(((p.M + 127) / 128) * p.H * p.B, 1, 1);
   switch (p.D) {
-    case 16: return launch(fa_bwd_dq_from_ds_kernel<T, 16>, grid, QdsCfg<T, 16>::LDS_BYTES, stream, p);
-    case 32: return launch(fa_bwd_dq_from_ds_kernel<T, 32>, grid, QdsCfg<T, 32>::LDS_BYTES, stream, p);
-    case 64: return launch(fa_bwd_dq_from_ds_kernel<T, 64>, grid, QdsCfg<T, 64>::LDS_BYTES, stream, p);
-    case 128: return launch(fa_bwd_dq_from_ds_kernel<T, 128>, grid, QdsCfg<T, 128>::LDS_BYTES, stream, p);
+    case 16: return launch(fa_bwd_dq_from_ds_kernel<T, 16, PW>, grid, QdsCfg<T, 16>::LDS_BYTES, stream, p);
+    case 32: return launch(fa_bwd_dq_from_ds_kernel<T, 32, PW>, grid, QdsCfg<T, 32>::LDS_BYTES, stream, p);
+    case 64: return launch(fa_bwd_dq_from_ds_kernel<T, 64, PW>, grid, QdsCfg<T, 64>::LDS_BYTES, stream, p);
+    case 128: return launch(fa_bwd_dq_from_ds_kernel<T, 128, PW>, grid, QdsCfg<T, 128>::LDS_BYTES, stream, p);
   }
   return kUnsupported;
 }
@@ -778,17 +797,21 @@ int64_t bwd_ds_workspace_bytes(int B, int H, int M, int N) {
   return (int64_t)B * H * (4 * (int64_t)((M + 127) / 128)) * (4 * (int64_t)((N + 127) / 128)) * 2048;
 }
 
-int run_bwd_dkdv_ds(const BwdParams& p, hipStream_t stream) {
-  if (!bwd_args_ok(p, false) || !dkdv_chunk_ok(p, false) || !p.ds) return kBadArgument;
-  if (p.dtype == kDtypeF16) return dispatch_dkdv<hw::half_t>(p, false, true, stream);
-  if (p.dtype == kDtypeBF16) return dispatch_dkdv<hw::bf16_t>(p, false, true, stream);
+int run_bwd_dkdv_ds(const BwdParams& p, bool piecewise, hipStream_t stream) {
+  if (!bwd_args_ok(p, piecewise) || !dkdv_chunk_ok(p, piecewise) || !p.ds) return kBadArgument;
+  if (p.dtype == kDtypeF16) return dispatch_dkdv<hw::half_t>(p, piecewise, true, stream);
+  if (p.dtype == kDtypeBF16) return dispatch_dkdv<hw::bf16_t>(p, piecewise, true, stream);
   return kUnsupported;
 }
 
-int run_bwd_dq_from_ds(const BwdParams& p, hipStream_t stream) {
+// piecewise: one launch per regime (p.regime, with p.k and p.dq set to that regime's tensors)
+int run_bwd_dq_from_ds(const BwdParams& p, bool piecewise, hipStream_t stream) {
   if (p.B <= 0 || p.H <= 0 || p.M <= 0 || p.N <= 0 || p.group <= 0 || !p.ds) return kBadArgument;
-  if (p.dtype == kDtypeF16) return launch_dq_from_ds<hw::half_t>(p, stream);
-  if (p.dtype == kDtypeBF16) return launch_dq_from_ds<hw::bf16_t>(p, stream);
+  if (piecewise && !(p.regime == 1 || p.regime == 2)) return kBadArgument;
+  if (p.dtype == kDtypeF16)
+    return piecewise ? launch_dq_from_ds<hw::half_t, true>(p, stream) : launch_dq_from_ds<hw::half_t, false>(p, stream);
+  if (p.dtype == kDtypeBF16)
+    return piecewise ? launch_dq_from_ds<hw::bf16_t, true>(p, stream) : launch_dq_from_ds<hw::bf16_t, false>(p, stream);
   return kUnsupported;
 }
 

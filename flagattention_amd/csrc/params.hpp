@@ -31,6 +31,8 @@ struct BwdParams {
   const float* lse;            // (B, H, M)
   float* delta;                // (B, H, M) rowsum(O * dO): written by the preprocess, read by the rest
   void* ds;                    // optional dS workspace: written by the dK/dV kernel, read by dQ-from-dS
+                               // (piecewise: the near regime's grid, then the far regime's)
+  int regime;                  // piecewise dQ-from-dS only: 1 = near entries (k = k1), 2 = far entries (k = k2)
   int B, H, M, N, D;
   int group;
   int chunk;  // query heads whose dK/dV one workgroup accumulates (divides group; 0 = group)
@@ -109,8 +111,8 @@ struct PagedParams {
 };
 
 int64_t bwd_ds_workspace_bytes(int B, int H, int M, int N);
-int run_bwd_dkdv_ds(const BwdParams& p, hipStream_t stream);
-int run_bwd_dq_from_ds(const BwdParams& p, hipStream_t stream);
+int run_bwd_dkdv_ds(const BwdParams& p, bool piecewise, hipStream_t stream);
+int run_bwd_dq_from_ds(const BwdParams& p, bool piecewise, hipStream_t stream);
 int run_splitkv(const SplitParams& p, hipStream_t stream);
 int run_combine(const CombineParams& p, hipStream_t stream);
 int run_paged(const PagedParams& p, hipStream_t stream);

@@ -170,14 +170,15 @@ def dkdv_heads_per_slice(B, H, group, N, num_cus):
 DS_WORKSPACE_LIMIT_MIB = int(os.environ.get("FLAGATTN_DS_WORKSPACE_MIB", "8192"))
 
 
-def ds_heads_per_launch(lib, B, H, group, M, N, D):
+def ds_heads_per_launch(lib, B, H, group, M, N, D, grids=1):
     """How many (batch, head) slices one dK/dV + dQ-from-dS launch pair may cover, 0 = recompute dS
-    in the dQ kernel instead.  Keeping dS costs M * N * 2 bytes per head, written once and read once;
-    it pays when the two recomputed products are expensive (head size 128) and the matrix is big
-    enough for the launches to fill the device."""
+    in the dQ kernel instead.  Keeping dS costs M * N * 2 bytes per head (times ``grids``: piecewise
+    attention keeps one grid per regime), written once and read once; it pays when the two recomputed
+    products are expensive (head size 128) and the matrix is big enough for the launches to fill the
+    device."""
     if D < 128 or M * N < 1024 * 1024 or DS_WORKSPACE_LIMIT_MIB <= 0:
         return 0
-    per_head = lib.fa_bwd_ds_workspace_mib(1, 1, M, N)
+    per_head = grids * lib.fa_bwd_ds_workspace_mib(1, 1, M, N)
     fit = DS_WORKSPACE_LIMIT_MIB // per_head
     if fit >= B * H:
         return B * H
@@ -185,10 +186,10 @@ def ds_heads_per_launch(lib, B, H, group, M, N, D):
     return fit
 
 
-def _ds_workspace(lib, device, B, H, M, N):
+def _ds_workspace(lib, device, B, H, M, N, grids=1):
     mib = lib.fa_bwd_ds_workspace_mib(B, H, M, N)
     assert mib > 0
-    return torch.empty(mib << 20, dtype=torch.uint8, device=device)
+    return torch.empty(grids * (mib << 20), dtype=torch.uint8, device=device)
 
 
 def attention(q, k, v, causal=False, sm_scale=None, dropout_p=0.0,

@@ -9,6 +9,7 @@ import math
 import torch
 
 from . import _abi, _lib
+from .flash import _ds_workspace, ds_heads_per_launch
 
 __all__ = ["attention"]
 
@@ -54,10 +55,29 @@ class PiecewiseAttention(torch.autograd.Function):
             dk1 = torch.empty(k1.shape, dtype=k1.dtype, device=k1.device)
             dk2 = torch.empty(k2.shape, dtype=k2.dtype, device=k2.device)
             dv = torch.empty(v.shape, dtype=v.dtype, device=v.device)
-            _abi.pw_bwd_dkdv(lib, q1, k1, q2, k2, v, do, L, delta, dk1, dk2, dv, ctx.w, ctx.causal, ctx.sm_scale)
             dq1 = torch.empty(q1.shape, dtype=q1.dtype, device=q1.device)
             dq2 = torch.empty(q2.shape, dtype=q2.dtype, device=q2.device)
-            _abi.pw_bwd_dq(lib, q1, k1, q2, k2, v, do, L, delta, dq1, dq2, ctx.w, ctx.causal, ctx.sm_scale)
+            B, H, M, D = q1.shape
+            N = k1.shape[2]
+            args = (ctx.w, ctx.causal, ctx.sm_scale)
+            # dS handed from the dK/dV kernel to the dQ kernels, one chunk grid per regime, when it pays
+            heads = ds_heads_per_launch(lib, B, H, 1, M, N, D, grids=2)
+            if heads == 0:
+                _abi.pw_bwd_dkdv(lib, q1, k1, q2, k2, v, do, L, delta, dk1, dk2, dv, *args)
+                _abi.pw_bwd_dq(lib, q1, k1, q2, k2, v, do, L, delta, dq1, dq2, *args)
+            elif heads >= B * H:
+                ds = _ds_workspace(lib, q1.device, B, H, M, N, grids=2)
+                _abi.pw_bwd_dkdv_ds(lib, q1, k1, q2, k2, v, do, L, delta, dk1, dk2, dv, ds, *args)
+                _abi.pw_bwd_dq_from_ds(lib, k1, k2, ds, dq1, dq2, *args)
+            else:  # bounded workspace: one batch entry and `heads` heads at a time
+                heads = min(heads, H)
+                ds = _ds_workspace(lib, q1.device, 1, heads, M, N, grids=2)
+                for b in range(B):
+                    for h0 in range(0, H, heads):
+                        s = (slice(b, b + 1), slice(h0, min(H, h0 + heads)))
+                        _abi.pw_bwd_dkdv_ds(lib, q1[s], k1[s], q2[s], k2[s], v[s], do[s], L[s], delta[s],
+                                            dk1[s], dk2[s], dv[s], ds, *args)
+                        _abi.pw_bwd_dq_from_ds(lib, k1[s], k2[s], ds, dq1[s], dq2[s], *args)
         return dq1, dk1, dq2, dk2, dv, None, None, None
 
 

@@ -139,6 +139,22 @@ int pw_bwd_dq(int dtype, const fa_view4* q1, const fa_view4* k1, const fa_view4*
               const float* delta, const fa_view4* dq1, const fa_view4* dq2, int B, int H, int M,
               int N, int D, int dist_threshold, int causal, float sm_scale, void* stream);
 
+/* pw_bwd_dkdv_ds + pw_bwd_dq_from_ds <- the same two reference kernels (piecewise.py:450-627 and
+ * :630-792) with dS handed over instead of recomputed, as fa_bwd_dkdv_ds / fa_bwd_dq_from_ds do for
+ * flash attention.  An entry of dS belongs to exactly one regime, so the workspace holds two chunk
+ * grids, the near regime's (q1.k1 entries, read for dq1 = dS k1) followed by the far regime's (read
+ * for dq2 = dS k2): at least 2 * fa_bwd_ds_workspace_mib(B, H, M, N) MiB, 16-byte aligned, contents
+ * on entry irrelevant.  pw_bwd_dq_from_ds launches one kernel per regime and must follow, on the same
+ * stream, the pw_bwd_dkdv_ds call with the same shape, dist_threshold and causal flag. */
+int pw_bwd_dkdv_ds(int dtype, const fa_view4* q1, const fa_view4* k1, const fa_view4* q2,
+                   const fa_view4* k2, const fa_view4* v, const fa_view4* dout, const float* lse,
+                   const float* delta, const fa_view4* dk1, const fa_view4* dk2, const fa_view4* dv,
+                   void* ds_workspace, int64_t ds_workspace_bytes, int B, int H, int M, int N, int D,
+                   int dist_threshold, int causal, float sm_scale, void* stream);
+int pw_bwd_dq_from_ds(int dtype, const fa_view4* k1, const fa_view4* k2, const void* ds_workspace,
+                      int64_t ds_workspace_bytes, const fa_view4* dq1, const fa_view4* dq2, int B, int H,
+                      int M, int N, int D, int dist_threshold, int causal, float sm_scale, void* stream);
+
 /* ---------------------------------------------------------------------------- paged attention --
  * paged_attn   <- `_paged_attn_kernel` (src/flag_attn/paged.py:204-349; launches :57-88, :112-142)
  * paged_reduce <- `_paged_attn_v2_reduce_kernel` (paged.py:352-435; launch :144-162)

@@ -82,3 +82,38 @@ def test_reduces_to_flash_when_threshold_is_out_of_range(causal):
     far = flag_attn.piecewise_attention(q1, k1, q2, k2, v, -900, causal=causal)
     check("near", near, oracle_flash(q1, k1, v, causal), oracle_flash(q1, k1, v, causal, upcast=True))
     check("far", far, oracle_flash(q2, k2, v, causal), oracle_flash(q2, k2, v, causal, upcast=True))
+
+
+@pytest.mark.parametrize("M,N,w,causal", [
+    (1100, 1300, 300, True),      # threshold inside blocks
+    (1024, 1024, 256, True),      # threshold on a block edge
+    (1200, 1100, 0, True),        # M > N: rows without keys; every visible pair far
+    (1100, 1300, -100, False),    # non-causal: future keys within 100 are far as well
+    (1100, 1300, 5000, False),    # every pair near: the far grid stays unread
+])
+def test_backward_with_stored_ds(monkeypatch, M, N, w, causal):
+    """Head size 128 and >= 2^20 scores: the dK/dV kernel leaves dS in a workspace (one chunk grid per
+    regime) for the dQ kernels.  Checked against the oracle, against the recomputing route, and with
+    a workspace bound that forces one (batch, head) slice per launch."""
+    from flagattention_amd import flash
+    B, H, D, dtype = 2, 2, 128, torch.bfloat16
+    ts = inputs(B, H, M, N, D, dtype, "BTHD", 1.0, True)
+    do = make((B, H, M, D), dtype, "BHTD", 1.0, 6)
+    assert flash.ds_heads_per_launch(flag_attn._lib.get(), B, H, 1, M, N, D, grids=2) >= B * H
+    g_ds = torch.autograd.grad(flag_attn.piecewise_attention(*ts, w, causal=causal), ts, do)
+    g_ref = torch.autograd.grad(oracle_pw(*ts, w, causal=causal, upcast=True), ts, do)
+    g_same = torch.autograd.grad(oracle_pw(*ts, w, causal=causal, upcast=False), ts, do)
+    for name, h, s, r in zip(("dq1", "dk1", "dq2", "dk2", "dv"), g_ds, g_same, g_ref):
+        assert not torch.isnan(h).any(), name
+        check(name, h, s, r)
+    per_slice = 2 * flag_attn._lib.get().fa_bwd_ds_workspace_mib(1, 1, M, N)
+    monkeypatch.setattr(flash, "DS_WORKSPACE_LIMIT_MIB", per_slice)
+    g_sliced = torch.autograd.grad(flag_attn.piecewise_attention(*ts, w, causal=causal), ts, do)
+    monkeypatch.setattr(flash, "DS_WORKSPACE_LIMIT_MIB", 0)
+    g_rec = torch.autograd.grad(flag_attn.piecewise_attention(*ts, w, causal=causal), ts, do)
+    for name, a, b, c in zip(("dq1", "dk1", "dq2", "dk2", "dv"), g_ds, g_sliced, g_rec):
+        assert torch.equal(a, b), name          # same kernels on slices
+        if name.startswith("dq"):  # same products and rounding; the summation order inside the MFMA differs
+            assert (a.float() - c.float()).abs().max() <= 2e-2 * c.float().abs().max() + 1e-6, name
+        else:
+            assert torch.equal(a, c), name

@@ -198,6 +198,7 @@ PW_CASES = [
     (1, 1, 140, 140, 16, 1000, True, torch.float16),    # every pair is near
     (1, 1, 70, 330, 32, -1000, False, torch.bfloat16),  # non-causal, every pair far
     (1, 1, 330, 70, 32, 129, False, torch.float16),     # M > N, threshold on a block edge
+    (2, 2, 200, 330, 128, 64, True, torch.bfloat16),    # head size 128, threshold on a block edge, two heads
 ]
 
 
@@ -223,6 +224,19 @@ def test_piecewise_forward_backward(lib, B, H, M, N, D, w, causal, dtype):
     check("o", o, same, ref)
     for name, h, s, r in zip(("dq1", "dk1", "dq2", "dk2", "dv"), (dq1, dk1, dq2, dk2, dv), g_same, g_ref):
         check(name, h, s, r)
+    # the same backward with dS handed over in the workspace (unwritten chunks hold NaN)
+    mib = lib.fa_bwd_ds_workspace_mib(B, H, M, N)
+    ds = torch.full((2 * (mib << 19),), float("nan"), dtype=dtype)
+    ek1, ek2, ev = (torch.full_like(d[1], float("nan")) for _ in range(3))
+    eq1, eq2 = (torch.full_like(d[0], float("nan")) for _ in range(2))
+    _abi.pw_bwd_dkdv_ds(lib, *d, do, lse, delta, ek1, ek2, ev, ds, w, causal, sc)
+    _abi.pw_bwd_dq_from_ds(lib, d[1], d[3], ds, eq1, eq2, w, causal, sc)
+    assert torch.equal(ek1, dk1) and torch.equal(ek2, dk2) and torch.equal(ev, dv)
+    assert not torch.isnan(eq1).any() and not torch.isnan(eq2).any()
+    check("dq1 from dS", eq1, g_same[0], g_ref[0])
+    check("dq2 from dS", eq2, g_same[2], g_ref[2])
+    for e, h in ((eq1, dq1), (eq2, dq2)):
+        assert (e.float() - h.float()).abs().max() <= 2e-2 * h.float().abs().max() + 1e-6
 
 
 SPLIT_CASES = [
