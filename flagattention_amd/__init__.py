@@ -7,5 +7,6 @@ from .flash import attention as flash_attention  # noqa: F401
 from .split_kv import attention as flash_attention_split_kv  # noqa: F401
 from .paged import attention as paged_attention  # noqa: F401
 from .total import total_attention  # noqa: F401
+from . import testing  # noqa: F401
 
 __version__ = "0.1.0"

@@ -171,6 +171,13 @@ def pw_bwd_dq_from_ds(lib, k1, k2, ds, dq1, dq2, w, causal, sm_scale):
                                 float(sm_scale), stream_of(dq1)), "pw_bwd_dq_from_ds")
 
 
+def fa_dropout_mask(lib, mask, dropout_p, seed, offset):
+    B, H, M, N = mask.shape
+    assert mask.is_contiguous() and mask.element_size() == 1
+    check(lib.fa_dropout_mask(ptr(mask), B, H, M, N, float(dropout_p), _u64(seed), _u64(offset),
+                              stream_of(mask)), "fa_dropout_mask")
+
+
 def fa_total_attn(lib, q, k, lse, total, causal, sm_scale):
     B, H, M, D = q.shape
     Hk, N = k.shape[1], k.shape[2]

@@ -34,6 +34,7 @@ SIGNATURES = {
     "fa_total_attn": [_i, _v, _v, _p, _p, _i, _i, _i, _i, _i, _i, _i, _f, _p],
     "fa_splitkv_fwd": [_i, _v, _v, _v, _p, _p, _i, _i, _i, _i, _i, _i, _i, _f, _i, _i, _p],
     "fa_splitkv_combine": [_i, _p, _p, _v, _p, _i, _i, _i, _i, _i, _p],
+    "fa_dropout_mask": [_p, _i, _i, _i, _i, _f, _u64, _u64, _p],
     "pw_fwd": [_i, _v, _v, _v, _v, _v, _v, _p, _i, _i, _i, _i, _i, _i, _i, _f, _p],
     "pw_bwd_dkdv": [_i, _v, _v, _v, _v, _v, _v, _p, _p, _v, _v, _v, _i, _i, _i, _i, _i, _i, _i, _f, _p],
     "pw_bwd_dq": [_i, _v, _v, _v, _v, _v, _v, _p, _p, _v, _v, _i, _i, _i, _i, _i, _i, _i, _f, _p],

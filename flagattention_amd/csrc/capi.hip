@@ -237,6 +237,16 @@ int pw_bwd_dq_from_ds(int dtype, const fa_view4* k1, const fa_view4* k2, const v
   return fa::run_bwd_dq_from_ds(p, true, (hipStream_t)stream);
 }
 
+int fa_dropout_mask(uint8_t* mask, int B, int H, int M, int N, float dropout_p, uint64_t seed,
+                    uint64_t offset, void* stream) {
+  if (B <= 0 || H <= 0 || M <= 0 || N <= 0) return FA_ERR_BAD_ARGUMENT;
+  fa::MaskParams p = {};
+  p.mask = mask;
+  p.total = (int64_t)B * H * M * N;
+  p.dropout_p = dropout_p; p.seed = seed; p.offset = offset;
+  return fa::run_dropout_mask(p, (hipStream_t)stream);
+}
+
 int fa_total_attn(int dtype, const fa_view4* q, const fa_view4* k, const float* lse, float* total,
                   int B, int H, int Hk, int M, int N, int D, int causal, float sm_scale,
                   void* stream) {

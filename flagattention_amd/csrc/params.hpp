@@ -110,6 +110,14 @@ struct PagedParams {
   float* ws; int num_wgs;
 };
 
+struct MaskParams {
+  uint8_t* mask;   // (B, H, M, N) contiguous, one byte per element: 1 = kept
+  int64_t total;   // B * H * M * N
+  float dropout_p;
+  uint64_t seed, offset;
+};
+int run_dropout_mask(const MaskParams& p, hipStream_t stream);
+
 int64_t bwd_ds_workspace_bytes(int B, int H, int M, int N);
 int run_bwd_dkdv_ds(const BwdParams& p, bool piecewise, hipStream_t stream);
 int run_bwd_dq_from_ds(const BwdParams& p, bool piecewise, hipStream_t stream);

@@ -14,6 +14,7 @@ from . import _abi, _lib
 from .split_kv import (num_splits_heuristic, split_kv_forward, SPLIT_BLOCK_M, SPLIT_BLOCK_N,
                        DECODE_MAX_ROWS)
 from .total import _total_attention
+from .dropout import philox_cuda_seed_offset
 
 __all__ = ["attention"]
 
@@ -57,7 +58,7 @@ class FlashAttention(torch.autograd.Function):
             num_cus = lib.fa_num_cus()
             is_dropout = dropout_p > 0
             if is_dropout:   # one Philox counter value per score element (flash.py:52-57)
-                seed, offset = philox_seed_offset(B * H * M * N, q.device)
+                seed, offset = philox_cuda_seed_offset(B * H * M * N, q.device)
             else:
                 seed, offset = 0, 0
             dropout = (dropout_p, seed, offset)
@@ -136,20 +137,6 @@ class FlashAttention(torch.autograd.Function):
                 dk = dk.reshape(B, Hk, slices // Hk, N, D).sum(2)
                 dv = dv.reshape(B, Hk, slices // Hk, N, D).sum(2)
         return dq, dk, dv, None, None, None, None, None, None
-
-
-def philox_seed_offset(increment, device):
-    """(seed, offset) of the device's default random generator, whose offset is then advanced by
-    ``increment`` rounded up to a multiple of 4 -- the generator state is two int64 words, seed and
-    offset, exactly as ``src/flag_attn/dropout.py:5-16`` of the reference reads and advances it."""
-    index = device.index if device.index is not None else torch.cuda.current_device()
-    gen = torch.cuda.default_generators[index]
-    state = gen.get_state()
-    words = state.view(torch.int64)
-    seed, offset = int(words[0]), int(words[1])
-    words[1] += (increment + 3) // 4 * 4
-    gen.set_state(state)
-    return seed, offset
 
 
 def dkdv_heads_per_slice(B, H, group, N, num_cus):

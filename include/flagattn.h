@@ -120,6 +120,12 @@ int fa_splitkv_fwd(int dtype, const fa_view4* q, const fa_view4* k, const fa_vie
 int fa_splitkv_combine(int dtype, const void* part_o, const float* part_lse, const fa_view4* o,
                        float* lse, int B, int H, int M, int D, int num_splits, void* stream);
 
+/* fa_dropout_mask <- `recompute_mask_kernel` (src/flag_attn/testing/dropout.py:5-25, launched by
+ * `recompute_mask`, :19-25): writes the (B, H, M, N) contiguous mask, one byte per element (1 = kept),
+ * that fa_fwd / fa_bwd_* apply for the same (dropout_p, seed, offset).  `mask` 16-byte aligned. */
+int fa_dropout_mask(uint8_t* mask, int B, int H, int M, int N, float dropout_p, uint64_t seed,
+                    uint64_t offset, void* stream);
+
 /* ------------------------------------------------------------------------ piecewise attention --
  * pw_fwd      <- piecewise `_fwd_kernel`    (src/flag_attn/piecewise.py:223-370, launch :50-69)
  * pw_bwd_dkdv <- piecewise `_bwd_kv_kernel` (piecewise.py:450-627, launch :114-139)

@@ -255,6 +255,40 @@ def test_attention_dropout(B, Hq, Hk, M, N, D, causal, dtype, dropout_p):
         check(name, h, s, r)
 
 
+@pytest.mark.parametrize("B,H,M,N", [(2, 4, 512, 612), (2, 4, 1024, 1034), (2, 4, 4001, 4096), (1, 2, 8192, 8202)])
+@pytest.mark.parametrize("p", [0.5, 0.8])
+def test_recompute_mask(B, H, M, N, p):
+    """flag_attn.testing.recompute_mask on the HIP kernel: drop rate within 1 % of p as the reference
+    asserts (tests/flag_attn/test_dropout.py:18-30), and bit-exact with the oracle's Philox restatement
+    on the first and the last rows of the tensor."""
+    from oracle import keep_mask
+    seed, offset = 123456789, 123456789123456789
+    mask = flag_attn.testing.recompute_mask(B, H, M, N, p, seed, offset, torch.cuda.current_device())
+    assert mask.dtype == torch.bool and mask.shape == (B, H, M, N)
+    dropped = (~mask).float().mean().item()
+    assert abs(dropped - p) < 0.01 * p
+    rows = 3
+    head = keep_mask(1, 1, rows, N, p, seed, offset, device="cuda")[0, 0]
+    assert torch.equal(mask[0, 0, :rows], head)
+    last = offset + ((B * H - 1) * M + (M - rows)) * N          # counter of element (B-1, H-1, M-rows, 0)
+    tail = keep_mask(1, 1, rows, N, p, seed, last, device="cuda")[0, 0]
+    assert torch.equal(mask[-1, -1, M - rows:], tail)
+    assert flag_attn.testing.recompute_mask(1, 1, 4, 4, 0.0, seed, offset, "cuda").all()
+
+
+def test_dropout_mask_matches_what_the_attention_kernels_drew():
+    """The reference's own dropout test (tests/flag_attn/test_flash_attention.py:225-262): rebuild the
+    mask from the returned (seed, offset) with recompute_mask and compare against the reference
+    computation with that mask."""
+    B, H, M, N, D, p = 2, 4, 512, 612, 64, 0.3
+    q, k, v = (make((B, H, T, D), torch.float16, "BHTD", 1.0, s) for T, s in ((M, 1), (N, 2), (N, 3)))
+    o, _, _, seed, offset = flag_attn.flash_attention(q, k, v, True, dropout_p=p, return_seed_offset=True)
+    mask = flag_attn.testing.recompute_mask(B, H, M, N, p, seed, offset, q.device)
+    ref = oracle_flash(q, k, v, True, upcast=True, dropout_p=p, dropout_mask=mask)
+    same = oracle_flash(q, k, v, True, upcast=False, dropout_p=p, dropout_mask=mask)
+    check("o", o, same, ref)
+
+
 def test_dropout_advances_the_generator_and_is_reproducible():
     q, k, v = (make((2, 16, 256, 64), torch.float16, "BHTD", 1.0, s) for s in (1, 2, 3))
     torch.cuda.manual_seed(4321)

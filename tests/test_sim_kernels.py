@@ -130,6 +130,20 @@ def test_flash_backward_with_stored_ds(lib, B, H, Hk, M, N, D, causal, dtype, bt
     assert (dq.float() - dq_plain.float()).abs().max() <= 2e-2 * dq_plain.float().abs().max() + 1e-6
 
 
+@pytest.mark.parametrize("B,H,M,N,pd,seed,offset", [
+    (1, 2, 7, 33, 0.3, 1234, 40),                                   # 462 elements: a vector tail
+    (2, 1, 16, 16, 0.5, 987654321987, 123456789123456789),          # 64-bit counter, whole vectors only
+    (1, 1, 3, 5, 0.9, 7, (1 << 32) - 4),                             # the counter's low word wraps
+])
+def test_dropout_mask_kernel_is_bit_exact_with_the_oracle(lib, B, H, M, N, pd, seed, offset):
+    """fa_dropout_mask (the reference's recompute_mask_kernel, testing/dropout.py:5-25) against the
+    numpy restatement of Triton's Philox in oracle/dropout.py."""
+    from oracle import keep_mask
+    mask = torch.zeros((B, H, M, N), dtype=torch.bool)
+    _abi.fa_dropout_mask(lib, mask, pd, seed, offset)
+    assert torch.equal(mask, keep_mask(B, H, M, N, pd, seed, offset))
+
+
 DROPOUT_CASES = [
     # B, H, Hk, M, N, D, causal, dtype, p, seed, offset
     (1, 2, 1, 70, 100, 64, True, torch.bfloat16, 0.3, 1234, 40),
