@@ -1,0 +1,82 @@
+"""Size-independent properties of the kernels at the benchmark's full sizes, where the fp32 oracle is
+too slow to cover every element: they hold exactly (bit for bit) by construction of the algorithm, so
+any indexing, masking or tile-ordering mistake that depends on the position in a large tensor breaks
+them.
+"""
+import pytest
+import torch
+
+import flagattention_amd as flag_attn
+
+pytestmark = pytest.mark.gpu
+
+B, H, T, D = 1, 32, 8192, 128
+
+
+def randn(shape, dtype, seed, grad=False):
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    t = torch.empty(shape, dtype=dtype, device="cuda").normal_(0.0, 1.0, generator=g)
+    return t.requires_grad_() if grad else t
+
+
+@pytest.fixture(scope="module")
+def full():
+    q, k, v = (randn((B, H, T, D), torch.bfloat16, s, grad=True) for s in (1, 2, 3))
+    do = randn((B, H, T, D), torch.bfloat16, 4)
+    o, L, tot, _, _ = flag_attn.flash_attention(q, k, v, causal=True, return_log_normalizer=True,
+                                                return_total_attention=True)
+    grads = torch.autograd.grad(o, (q, k, v), do, retain_graph=True)
+    return q, k, v, do, o, L, tot, grads
+
+
+def test_backward_is_exactly_linear_under_a_power_of_two(full):
+    """dO -> 2 dO doubles delta, dP and dS exactly and commutes with every rounding to bf16, so every
+    gradient doubles bit for bit (the dS-kept route at this size)."""
+    q, k, v, do, o, _, _, grads = full
+    doubled = torch.autograd.grad(o, (q, k, v), 2 * do, retain_graph=True)
+    for name, g, g2 in zip(("dq", "dk", "dv"), grads, doubled):
+        assert torch.equal(2 * g, g2), name
+
+
+def test_heads_are_independent(full):
+    """A head computed alone, through strided views of the full tensors, equals the same head computed
+    in the full launch: forward outputs and all gradients, bit for bit."""
+    q, k, v, do, o, L, tot, grads = full
+    for h in (0, 13, 31):
+        hs = slice(h, h + 1)
+        qs, ks, vs = (t.detach()[:, hs].requires_grad_() for t in (q, k, v))
+        o1, L1, tot1, _, _ = flag_attn.flash_attention(qs, ks, vs, causal=True, return_log_normalizer=True,
+                                                       return_total_attention=True)
+        g1 = torch.autograd.grad(o1, (qs, ks, vs), do[:, hs])
+        assert torch.equal(o1, o[:, hs]) and torch.equal(L1, L[:, hs]) and torch.equal(tot1, tot[:, hs])
+        for name, a, b in zip(("dq", "dk", "dv"), g1, grads):
+            assert torch.equal(a, b[:, hs]), (name, h)
+
+
+def test_causal_prefix(full):
+    """With the causal mask and equal lengths, the first T' rows of the output depend on the first T'
+    keys only and walk the same tiles in the same order: truncating the sequence changes nothing."""
+    q, k, v, _, o, L, _, _ = full
+    for t in (128, 1000, 4097):
+        o1, L1, _, _, _ = flag_attn.flash_attention(q.detach()[:, :, :t], k.detach()[:, :, :t], v.detach()[:, :, :t],
+                                                    causal=True, return_log_normalizer=True)
+        assert torch.equal(o1, o[:, :, :t]) and torch.equal(L1, L[:, :, :t]), t
+
+
+def test_total_attention_sums_to_the_number_of_rows(full):
+    """Every query row distributes a total probability of 1 over the keys."""
+    _, _, _, _, _, _, tot, _ = full
+    sums = tot.double().sum(-1)
+    assert torch.allclose(sums, torch.full_like(sums, float(T)), rtol=2e-3)
+    assert (tot >= 0).all()
+
+
+def test_log_normalizer_bounds(full):
+    """L = logsumexp of the visible scaled scores: at least the largest of them (row m's own key m is
+    visible) and at most that maximum plus log(number of visible keys)."""
+    q, k, _, _, _, L, _, _ = full
+    m = torch.arange(T, device="cuda")
+    own = (q.detach().float() * k.detach().float()).sum(-1) * D ** -0.5     # score of (m, m)
+    assert (L >= own - 1e-2).all()
+    assert (L[:, :, 0] - own[:, :, 0]).abs().max() < 2e-2                      # row 0 sees one key
+    assert torch.isfinite(L).all() and m.numel() == L.shape[-1]
