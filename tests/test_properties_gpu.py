@@ -80,3 +80,49 @@ def test_log_normalizer_bounds(full):
     assert (L >= own - 1e-2).all()
     assert (L[:, :, 0] - own[:, :, 0]).abs().max() < 2e-2                      # row 0 sees one key
     assert torch.isfinite(L).all() and m.numel() == L.shape[-1]
+
+
+def test_offsets_beyond_two_to_the_31_elements():
+    """Tensors with more than 2^31 elements (batch 66 of the benchmark shape; 4.4 GB each): the last
+    (batch, head) slice, whose element offsets need 64 bits, equals the same slice computed alone --
+    forward, log-normalizer and all gradients (the backward runs in bounded-workspace slices)."""
+    Bb = 66
+    assert Bb * H * T * D > 2 ** 31
+    q, k, v = (randn((Bb, H, T, D), torch.bfloat16, s, grad=True) for s in (11, 12, 13))
+    do = randn((Bb, H, T, D), torch.bfloat16, 14)
+    o, L, _, _, _ = flag_attn.flash_attention(q, k, v, causal=True, return_log_normalizer=True)
+    dq, dk, dv = torch.autograd.grad(o, (q, k, v), do)
+    s = (slice(Bb - 1, Bb), slice(H - 1, H))
+    qs, ks, vs = (t.detach()[s].requires_grad_() for t in (q, k, v))
+    o1, L1, _, _, _ = flag_attn.flash_attention(qs, ks, vs, causal=True, return_log_normalizer=True)
+    g1 = torch.autograd.grad(o1, (qs, ks, vs), do[s])
+    assert torch.equal(o1, o[s]) and torch.equal(L1, L[s])
+    for name, a, b in zip(("dq", "dk", "dv"), g1, (dq, dk, dv)):
+        assert torch.equal(a, b[s]), name
+    assert torch.isfinite(o.float()).all()
+
+
+def test_paged_cache_beyond_two_to_the_31_elements():
+    """A key/value cache of 2.3 G elements per tensor, the sequences' blocks taken from its top end:
+    block offsets need 64 bits.  Compared with the same blocks copied into a small cache."""
+    num_blocks, hkv, bs, Dh, hq, num_seqs, ctx = 140000, 8, 16, 128, 32, 8, 2000
+    assert num_blocks * hkv * bs * Dh > 2 ** 31
+    g = torch.Generator(device="cuda").manual_seed(5)
+    kc = torch.empty((num_blocks, hkv, bs, Dh), dtype=torch.float16, device="cuda")
+    vc = torch.empty_like(kc)
+    per_seq = (ctx + bs - 1) // bs
+    used = num_seqs * per_seq
+    top = slice(num_blocks - used, num_blocks)
+    kc[top].normal_(0.0, 1.0, generator=g)
+    vc[top].normal_(0.0, 1.0, generator=g)
+    q = randn((num_seqs, hq, Dh), torch.float16, 6)
+    lens = torch.randint(1, ctx, (num_seqs,), dtype=torch.int32, device="cuda", generator=g)
+    lens[0] = ctx
+    perm = torch.randperm(used, device="cuda", generator=g)
+    table_small = perm.reshape(num_seqs, per_seq).int()
+    table_big = (table_small.long() + (num_blocks - used))
+    for splits in (0, 1, 4):
+        big = flag_attn.paged_attention(q, kc, vc, lens, table_big, Dh ** -0.5, ctx, num_splits=splits)
+        small = flag_attn.paged_attention(q, kc[top].contiguous(), vc[top].contiguous(), lens, table_small,
+                                          Dh ** -0.5, ctx, num_splits=splits)
+        assert torch.equal(big, small), splits
