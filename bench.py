@@ -276,7 +276,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (every (batch, head) slice "
-                 "is independent; see DESIGN.md for how it would shard). Run with --gpus 1.")
+                 "is independent and would shard over batch or heads with no exchange). Run with --gpus 1.")
     import torch
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU: the kernels have no CPU fallback")

@@ -88,7 +88,7 @@ def test_bfloat16_and_large_group():
 
 
 def test_baseline_decode_configuration_small_copy():
-    """The BASELINE decode configuration (32 query heads over 8 kv heads, head 128, block 16) at a
+    """The benchmark's decode configuration (32 query heads over 8 kv heads, head 128, block 16) at a
     reduced number of sequences so that the token-gather oracle stays fast."""
     run_case(8, 32, 4, 128, 16, 8192)
 
