@@ -221,6 +221,45 @@ def splitkv_bench(torch, iters=50):
                          "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None}}
 
 
+def piecewise_bench(torch, iters=10):
+    """piecewise_attention forward + backward, causal bf16 B=2 H=32 T=4096 D=128, threshold 1024.
+    FLOPs counted as for flash attention (one dot product per score), not with the reference's
+    1.5x / 1.6x convention for its two score products (benchmark/piecewise_benchmark.py:98-110)."""
+    import flagattention_amd as flag_attn
+    dev = "cuda:0"
+    g = torch.Generator(device=dev).manual_seed(10086)
+    B, H, T, D, w = 2, 32, 4096, 128, 1024
+    ts = [torch.randn(B, H, T, D, device=dev, dtype=torch.bfloat16, generator=g).requires_grad_() for _ in range(5)]
+    do = torch.randn(B, H, T, D, device=dev, dtype=torch.bfloat16, generator=g)
+    ms_fwd = timed_launches(lambda: flag_attn.piecewise_attention(*ts, w, causal=True), iters, torch)
+    o = flag_attn.piecewise_attention(*ts, w, causal=True)
+    ms_bwd = timed_launches(lambda: torch.autograd.grad(o, ts, do, retain_graph=True), iters, torch)
+    fwd = 4.0 * B * H * causal_pairs(T, T) * D
+    tf = (fwd * 3.5) / ((ms_fwd + ms_bwd) * 1e-3) / 1e12
+    return {"workload": "piecewise_attention fwd+bwd causal bf16 B=2 H=32 T=4096 D=128 dist_threshold=1024",
+            "ms_fwd": round(ms_fwd, 4), "ms_bwd": round(ms_bwd, 4), "counted_gflop": round(fwd * 3.5 / 1e9, 2),
+            "value": round(tf, 1), "unit": "TFLOP/s",
+            "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                         "frac": round(tf / PEAK_BF16_TFLOPS, 4), "traffic": None}}
+
+
+def total_attention_bench(torch, iters=20):
+    """total_attention (column sums of P) at the benchmark shape: one product, 2 * pairs * D per head."""
+    import flagattention_amd as flag_attn
+    dev = "cuda:0"
+    g = torch.Generator(device=dev).manual_seed(10086)
+    B, H, T, D = 1, 32, 8192, 128
+    q, k, v = (torch.randn(B, H, T, D, device=dev, dtype=torch.bfloat16, generator=g) for _ in range(3))
+    _, L, _, _, _ = flag_attn.flash_attention(q, k, v, causal=True, return_log_normalizer=True)
+    ms = timed_launches(lambda: flag_attn.total_attention(q, k, L, True, D ** -0.5), iters, torch)
+    flop = 2.0 * B * H * causal_pairs(T, T) * D
+    tf = flop / (ms * 1e-3) / 1e12
+    return {"workload": "total_attention causal bf16 B=1 H=32 T=8192 D=128", "ms": round(ms, 4),
+            "counted_gflop": round(flop / 1e9, 2), "value": round(tf, 1), "unit": "TFLOP/s",
+            "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                         "frac": round(tf / PEAK_BF16_TFLOPS, 4), "traffic": None}}
+
+
 def profile_kernel(args, torch):
     """A handful of launches of one kernel at the benchmark's shapes, nothing else on the device."""
     from flagattention_amd import _abi, _lib
@@ -298,6 +337,8 @@ def main():
     if not args.no_paged:
         out["paged_decode"] = paged_bench(torch)
         out["splitkv_decode"] = splitkv_bench(torch)
+        out["piecewise"] = piecewise_bench(torch)
+        out["total_attention"] = total_attention_bench(torch)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args, torch)
     print(json.dumps(out))
