@@ -99,3 +99,21 @@ def test_dtype_codes():
     assert _abi.dtype_code(torch.zeros(1, dtype=torch.bfloat16)) == 1
     with pytest.raises(AssertionError):
         _abi.dtype_code(torch.zeros(1, dtype=torch.float32))
+
+
+def test_reference_package_name_resolves_to_this_implementation():
+    """``import flag_attn`` and its submodules (the names the reference's callers use,
+    src/flag_attn/__init__.py:9-14) resolve to this package; nothing here needs a GPU."""
+    import flag_attn
+    import flag_attn.flash
+    import flag_attn.testing
+    from flag_attn.dropout import philox_cuda_seed_offset
+    from flag_attn.testing import recompute_mask
+    import flagattention_amd
+    assert flag_attn.flash_attention is flagattention_amd.flash_attention
+    assert flag_attn.piecewise_attention is flagattention_amd.piecewise_attention
+    assert flag_attn.paged_attention is flagattention_amd.paged_attention
+    assert flag_attn.flash_attention_split_kv is flagattention_amd.flash_attention_split_kv
+    assert flag_attn.flash is flagattention_amd.flash and flag_attn.testing is flagattention_amd.testing
+    assert callable(philox_cuda_seed_offset) and callable(recompute_mask)
+    assert callable(flag_attn.flash.get_fwd_config) and callable(flag_attn.flash.get_bwd_config)
