@@ -571,7 +571,9 @@ template <class T, int D>
 struct QdsCfg {
   static constexpr int BM = 128, BN = 64;
   static constexpr int DV = D < 32 ? 32 : D;
-  static constexpr int LD = DV + (DV == 128 ? 24 : 40);
+  // the K tile is only read through transposing reads: at head size 128, 64 B of padding keep the 4 rows x 2 halves
+  // that 32 lanes touch in disjoint banks (with the 48 B of the other backward tiles the two halves collide)
+  static constexpr int LD = DV + (DV == 128 ? 32 : 40);
   static constexpr int TILE = BN * LD;                 // K tile, elements
   static constexpr int VEC = 512 + 32 + 32;            // one chunk vector in the patch: 2 x (256 + 32 pad) elements
   static constexpr int PATCH = 2 * 2 * VEC;            // 2 chunks x 2 vectors per wavefront and stage
