@@ -26,6 +26,11 @@ randomized three-way comparison), see ``tests/test_oracle_*.py``:
   the Random123 known-answer vectors, the uniform map against its defining properties, the drop
   rate; dropout with an all-true mask equals no dropout; a hand-built mask against an explicit loop.
 
+All three operators are also held against fixed vectors (``tests/golden/attention_vectors.npz``, written by
+``tests/golden/make_vectors.py`` from scalar fp64 loops that state the definitions directly): bottom-right
+causal alignment with grouped heads, rows without keys, the piecewise distance rule, the paged block
+table (``tests/test_golden.py``; the same vectors check the kernels in the simulator and on the GPU).
+
 No function of this oracle is "parity unpinned" with respect to what the kernels are compared
 against.  One statement is: that ``dropout.keep_mask`` reproduces, bit for bit, the mask a Triton run
 of the reference would draw -- it restates Triton's published ``tl.rand`` but no such run is possible
