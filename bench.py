@@ -297,6 +297,13 @@ def profile_kernel(args, torch):
     for _ in range(5):
         fn()
     torch.cuda.synchronize()
+    if args.hold_seconds > 0:   # keep the kernel running back to back, e.g. to read the clock it settles at
+        import time
+        t0 = time.time()
+        while time.time() - t0 < args.hold_seconds:
+            for _ in range(50):
+                fn()
+            torch.cuda.synchronize()
     print(json.dumps({"profiled": args.profile_kernel, "workload": w["name"]}))
 
 
@@ -311,6 +318,8 @@ def main():
                                                   "paged_attn", "copy"],
                     help="run only this launch a few times (for rocprofv3 counter passes); 'copy' is a plain "
                          "1 GiB device copy used to calibrate FETCH_SIZE / WRITE_SIZE")
+    ap.add_argument("--hold-seconds", type=float, default=0.0,
+                    help="with --profile-kernel: afterwards repeat the launch for this long")
     ap.add_argument("--no-paged", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
