@@ -77,6 +77,8 @@ struct KvCfg {
   static constexpr int TILE = BM * LD;
   // register budget: two wavefronts per SIMD (256 registers each) when the accumulators allow it
   static constexpr int WAVES_PER_SIMD = D <= 64 ? 2 : 1;
+  // one wavefront per SIMD: overlap of matrix and element-wise work has to come from the instruction order
+  static constexpr bool SLOTTED = WAVES_PER_SIMD == 1 && BM == 64 && D == 128;
   static constexpr size_t STAGE_BYTES = 2 * TILE * sizeof(T) + 2 * BM * sizeof(float);  // Q, dO, L, delta
   static constexpr size_t LDS_BYTES = 2 * STAGE_BYTES;
 };
@@ -255,6 +257,109 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
       const float* sL = (const float*)(base + 2 * C::TILE * sizeof(T));
       const float* sDl = sL + C::BM;
 
+      // Tiles that no mask touches (all but the one or two on the diagonal), with one wavefront per
+      // SIMD: nothing else would issue under this wavefront's matrix instructions, so the
+      // element-wise work of one 32 x 32 block is written BETWEEN the matrix instructions of the
+      // other, one element per matrix instruction, in the order
+      //   A0 | A1 with E0 | C0 with E1 | C1      (A: S and dP, E: P and dS, C: dV and dK)
+      // and a scheduling fence after every such slot keeps the compiler from regrouping them.
+      bool plain_tile = false;
+      if constexpr (C::SLOTTED && !PW && !DROP) plain_tile = !p.causal || (m0 + pseq >= nw + 31);
+      if constexpr (C::SLOTTED && !PW && !DROP) {
+      if (plain_tile) {
+        constexpr int NA = 2 * C::KSTEPS;       // matrix instructions of an A phase (16)
+        constexpr int NC = 4 * (C::DV / 32);    // of a C phase (16)
+        static_assert(NA == 16 && NC == 16, "one element of a block per matrix instruction");
+        f32x16 sx[2], dpx[2], prx[2], dsx[2];
+        // operand of A-phase instruction j of block sb, and of C-phase instruction j
+        auto a_operand = [&](int sb, int j) {
+          return operand_rowmajor<T, C::LD>(j < C::KSTEPS ? sQ : sG, sb * 32, 16 * (j % C::KSTEPS), lane);
+        };
+        auto c_operand = [&](int sb, int j) {   // j = 8 c + 4 which + db
+          return operand_transposed<T, C::LD>((j & 4) ? sQ : sG, sb * 32 + 16 * (j >> 3), (j & 3) * 32, lane);
+        };
+        auto a_issue = [&](int sb, int j, const V8& op) {
+          if (j < C::KSTEPS) sx[sb] = hw::mfma32(op, kreg[j], sx[sb]);
+          else dpx[sb] = hw::mfma32(op, vreg[j - C::KSTEPS], dpx[sb]);
+        };
+        hw::f32x4 lrow[4], drow[4];
+        auto load_rows_stats = [&](int sb) {
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            lrow[g] = *(const hw::f32x4*)(sL + sb * 32 + 8 * g + 4 * hh);
+            drow[g] = *(const hw::f32x4*)(sDl + sb * 32 + 8 * g + 4 * hh);
+          }
+        };
+        auto element = [&](int sb, int r) {
+          const float pv = hw::exp2_fast(fmaf(sx[sb][r], c2, -lrow[r >> 2][r & 3]));
+          prx[sb][r] = pv;
+          dsx[sb][r] = pv * (dpx[sb][r] - drow[r >> 2][r & 3]);
+        };
+#pragma unroll
+        for (int sb = 0; sb < 2; ++sb)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) { sx[sb][r] = 0.f; dpx[sb][r] = 0.f; }
+
+        // ---- A0 ----
+#pragma unroll
+        for (int j = 0; j < NA; ++j) a_issue(0, j, a_operand(0, j));
+        hw::sched_prefetched_operands<NA, 8>();
+        hw::sched_fence();
+
+        // ---- A1 with E0 ----
+        constexpr int kDepthA = 4;
+        V8 ring_a[kDepthA];
+        load_rows_stats(0);
+#pragma unroll
+        for (int j = 0; j < kDepthA; ++j) ring_a[j] = a_operand(1, j);
+        hw::sched_fence();
+#pragma unroll
+        for (int j = 0; j < NA; ++j) {
+          a_issue(1, j, ring_a[j % kDepthA]);
+          if (j + kDepthA < NA) ring_a[j % kDepthA] = a_operand(1, j + kDepthA);
+          element(0, j);
+          hw::sched_fence();
+        }
+
+        // ---- C0 with E1 ----
+        constexpr int kDepthC = 3;
+        V8 ring_c[kDepthC];
+        V8 pa[2], da[2];
+#pragma unroll
+        for (int c = 0; c < 2; ++c) { pa[c] = pack_half_block<T>(prx[0], c); da[c] = pack_half_block<T>(dsx[0], c); }
+        load_rows_stats(1);
+#pragma unroll
+        for (int j = 0; j < kDepthC; ++j) ring_c[j] = c_operand(0, j);
+        hw::sched_fence();
+#pragma unroll
+        for (int j = 0; j < NC; ++j) {
+          const int c = j >> 3, db = j & 3;
+          if (j & 4) dk[db] = hw::mfma32(da[c], ring_c[j % kDepthC], dk[db]);
+          else dv[db] = hw::mfma32(pa[c], ring_c[j % kDepthC], dv[db]);
+          if (j + kDepthC < NC) ring_c[j % kDepthC] = c_operand(0, j + kDepthC);
+          if (DS && (j & 7) == 0)
+            hw::store_streaming(ds_row + (int64_t)(m0 / 32) * 1024 + c * 512, __builtin_bit_cast(u32x4, da[c]));
+          element(1, j);
+          hw::sched_fence();
+        }
+
+        // ---- C1 ----
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+          V8 pa1 = pack_half_block<T>(prx[1], c);
+#pragma unroll
+          for (int db = 0; db < C::DV / 32; ++db)
+            dv[db] = hw::mfma32(pa1, operand_transposed<T, C::LD>(sG, 32 + 16 * c, db * 32, lane), dv[db]);
+          V8 da1 = pack_half_block<T>(dsx[1], c);
+          if (DS) hw::store_streaming(ds_row + (int64_t)(m0 / 32 + 1) * 1024 + c * 512, __builtin_bit_cast(u32x4, da1));
+#pragma unroll
+          for (int db = 0; db < C::DV / 32; ++db)
+            dk[db] = hw::mfma32(da1, operand_transposed<T, C::LD>(sQ, 32 + 16 * c, db * 32, lane), dk[db]);
+        }
+        hw::sched_prefetched_operands<NC, 5, 2>();
+      }
+      }
+      if (!plain_tile) {
 #pragma unroll
       for (int sb = 0; sb < C::BM / 32; ++sb) {
         const int mr0 = m0 + sb * 32;
@@ -327,6 +432,7 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
         }
         // each of these products takes an operand made of two transposing reads
         hw::sched_prefetched_operands<4 * (C::DV / 32), (C::DV >= 128 ? 5 : 1), 2>();
+      }
       }
 
       if (more) commit(stage ^ 1);
