@@ -163,6 +163,11 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
   gr.init(tid, p.dout.st);
   float l_reg = 0.f, d_reg = 0.f;
   int l_row = 0;
+  // In the instantiation with the slot-structured body, LDS holds -L / sm_scale and -delta per row:
+  // the score and dP accumulators start from them, so that P = exp2(c2 (q.k - L / sm_scale)) and
+  // dS = P (dO.v - delta) take one multiplication each in the slots.
+  constexpr bool FOLDED = C::SLOTTED && !PW && !DROP;
+  const float inv_scale = 1.f / p.sm_scale;
   auto fetch = [&](int m0) {
     const int rows = M - m0;
     qr.fetch(q_src + (int64_t)m0 * q_stride, rows);
@@ -182,8 +187,13 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
     float* f = (float*)(base + 2 * C::TILE * sizeof(T));
     // rows past M get L = +inf, hence P = 0
     if (tid < C::BM) {
-      f[tid] = l_row < M ? l_reg * kLog2e : __builtin_inff();
-      f[C::BM + tid] = l_row < M ? d_reg : 0.f;
+      if constexpr (FOLDED) {  // what the accumulators of q.k and dO.v start from
+        f[tid] = l_row < M ? -l_reg * inv_scale : -__builtin_inff();
+        f[C::BM + tid] = l_row < M ? -d_reg : 0.f;
+      } else {
+        f[tid] = l_row < M ? l_reg * kLog2e : __builtin_inff();
+        f[C::BM + tid] = l_row < M ? d_reg : 0.f;
+      }
     }
   };
 
@@ -291,25 +301,27 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
           }
         };
         auto element = [&](int sb, int r) {
-          const float pv = hw::exp2_fast(fmaf(sx[sb][r], c2, -lrow[r >> 2][r & 3]));
+          const float pv = hw::exp2_fast(sx[sb][r] * c2);
           prx[sb][r] = pv;
-          dsx[sb][r] = pv * (dpx[sb][r] - drow[r >> 2][r & 3]);
+          dsx[sb][r] = pv * dpx[sb][r];
         };
+        auto start_block = [&](int sb) {   // accumulators start from the per-row values
+          load_rows_stats(sb);
 #pragma unroll
-        for (int sb = 0; sb < 2; ++sb)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) { sx[sb][r] = 0.f; dpx[sb][r] = 0.f; }
+          for (int r = 0; r < 16; ++r) { sx[sb][r] = lrow[r >> 2][r & 3]; dpx[sb][r] = drow[r >> 2][r & 3]; }
+        };
 
         // ---- A0 ----
+        start_block(0);
 #pragma unroll
         for (int j = 0; j < NA; ++j) a_issue(0, j, a_operand(0, j));
-        hw::sched_prefetched_operands<NA, 8>();
+        hw::sched_prefetched_operands<NA, 8, 1, 8>();
         hw::sched_fence();
 
         // ---- A1 with E0 ----
         constexpr int kDepthA = 4;
         V8 ring_a[kDepthA];
-        load_rows_stats(0);
+        start_block(1);
 #pragma unroll
         for (int j = 0; j < kDepthA; ++j) ring_a[j] = a_operand(1, j);
         hw::sched_fence();
@@ -327,7 +339,6 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
         V8 pa[2], da[2];
 #pragma unroll
         for (int c = 0; c < 2; ++c) { pa[c] = pack_half_block<T>(prx[0], c); da[c] = pack_half_block<T>(dsx[0], c); }
-        load_rows_stats(1);
 #pragma unroll
         for (int j = 0; j < kDepthC; ++j) ring_c[j] = c_operand(0, j);
         hw::sched_fence();
@@ -393,7 +404,8 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
             const int m = mr0 + block_row(r, hh);
             bool keep = !p.causal || (m + pseq >= my_n);
             if (PW) keep = keep && ((m + pseq - my_n >= p.w) == far_phase);
-            float pv = hw::exp2_fast(fmaf(s[r], c2, -lrow[r >> 2][r & 3]));
+            float pv = FOLDED ? hw::exp2_fast((s[r] + lrow[r >> 2][r & 3]) * c2)
+                              : hw::exp2_fast(fmaf(s[r], c2, -lrow[r >> 2][r & 3]));
             pv = keep ? pv : 0.f;
             float pd = pv, dpv = dp[r];
             if (DROP) {
@@ -402,12 +414,13 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
               dpv = kd ? dp[r] * rp : 0.f;
             }
             pr[r] = pd;
-            ds[r] = pv * (dpv - drow[r >> 2][r & 3]);
+            ds[r] = FOLDED ? pv * (dpv + drow[r >> 2][r & 3]) : pv * (dpv - drow[r >> 2][r & 3]);
           }
         } else {
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
-            const float pv = hw::exp2_fast(fmaf(s[r], c2, -lrow[r >> 2][r & 3]));
+            const float pv = FOLDED ? hw::exp2_fast((s[r] + lrow[r >> 2][r & 3]) * c2)
+                                    : hw::exp2_fast(fmaf(s[r], c2, -lrow[r >> 2][r & 3]));
             float pd = pv, dpv = dp[r];
             if (DROP) {
               const bool kd = dropout_keeps(drop_col + (uint64_t)(mr0 + block_row(r, hh)) * N, p.seed, p.dropout_p);
@@ -415,7 +428,7 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
               dpv = kd ? dp[r] * rp : 0.f;
             }
             pr[r] = pd;
-            ds[r] = pv * (dpv - drow[r >> 2][r & 3]);
+            ds[r] = FOLDED ? pv * (dpv + drow[r >> 2][r & 3]) : pv * (dpv - drow[r >> 2][r & 3]);
           }
         }
 #pragma unroll

@@ -109,9 +109,10 @@ FA_DEVICE void sched_fence() { __builtin_amdgcn_sched_barrier(0); }
 
 // Scheduling hint for a region of N matrix instructions that each consume an operand fetched by RPM
 // LDS reads: keep the operands of DEPTH matrix instructions in flight ahead of their consumer.
-template <int N, int DEPTH, int RPM = 1>
+// EXTRA other LDS reads precede the first operand read.
+template <int N, int DEPTH, int RPM = 1, int EXTRA = 0>
 FA_DEVICE void sched_prefetched_operands() {
-  __builtin_amdgcn_sched_group_barrier(0x100, DEPTH * RPM, 0);
+  __builtin_amdgcn_sched_group_barrier(0x100, DEPTH * RPM + EXTRA, 0);
 #pragma unroll
   for (int i = 0; i < N - DEPTH; ++i) {
     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);

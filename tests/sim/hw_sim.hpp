@@ -258,7 +258,7 @@ inline bool wave_any(bool pred) {
 
 inline void sched_fence() {}
 inline void keep_branch() {}
-template <int N, int DEPTH, int RPM = 1> inline void sched_prefetched_operands() {}
+template <int N, int DEPTH, int RPM = 1, int EXTRA = 0> inline void sched_prefetched_operands() {}
 inline float exp2_fast(float x) { return exp2f(x); }
 inline float log_nat(float x) { return logf(x); }
 

@@ -172,8 +172,8 @@ def _grads(q, k, v, do, causal):
 @pytest.mark.parametrize("Hk", [8, 2])
 def test_backward_with_bounded_ds_workspace_matches_unbounded(Hk, monkeypatch):
     """Head size 128 keeps dS in a workspace for the dQ kernel; with a small limit the backward walks
-    the batch and the heads in slices.  Both must give the very same bits, and the same dQ as the
-    kernel that recomputes dS (limit 0)."""
+    the batch and the heads in slices.  Both must give the very same bits; dK and dV also equal those
+    of the route that recomputes dS (limit 0), whose dQ agrees to rounding."""
     from flagattention_amd import flash as flash_mod
     q = make((2, 8, 1024, 128), torch.bfloat16, "BTHD", 1.0, 1, grad=True)
     k = make((2, Hk, 1100, 128), torch.bfloat16, "BTHD", 1.0, 2, grad=True)
@@ -189,14 +189,20 @@ def test_backward_with_bounded_ds_workspace_matches_unbounded(Hk, monkeypatch):
     monkeypatch.setattr(flash_mod, "DS_WORKSPACE_LIMIT_MIB", 0)
     assert flash_mod.ds_heads_per_launch(lib, 2, 8, 8 // Hk, 1024, 1100, 128) == 0
     recomputed = _grads(q, k, v, do, True)
-    for a, b, c in zip(whole, sliced, recomputed):
-        assert torch.equal(a, b) and torch.equal(a, c)
+    for name, a, b, c in zip(("o", "dq", "dk", "dv"), whole, sliced, recomputed):
+        assert torch.equal(a, b), name
+        if name == "dq":   # same products and the same rounding of dS to bf16, but P (dP - delta) is formed with
+            # delta folded into the dP accumulator in one kernel and subtracted afterwards in the other
+            assert (a.float() - c.float()).abs().max() <= 2e-2 * c.float().abs().max() + 1e-6
+        else:
+            assert torch.equal(a, c), name
 
 
 def test_full_size_backward_paths_agree():
     """The benchmark's shape (1 x 32 heads x 8192 x 128, causal, bf16) is too large for the fp32
-    oracle over all heads; what does not depend on size: dQ from the stored dS equals dQ from the
-    recomputed dS bit for bit, gradients are linear in dO, and 2 heads are checked against the oracle."""
+    oracle over all heads; what does not depend on size: dK and dV of the two backward routes are equal
+    bit for bit and dQ from the stored dS agrees with dQ from the recomputed dS to rounding, gradients are
+    linear in dO, and 2 heads are checked against the oracle."""
     from flagattention_amd import flash as flash_mod
     q = make((1, 32, 8192, 128), torch.bfloat16, "BHTD", 1.0, 1, grad=True)
     k = make((1, 32, 8192, 128), torch.bfloat16, "BHTD", 1.0, 2, grad=True)
@@ -212,8 +218,11 @@ def test_full_size_backward_paths_agree():
         recomputed = _grads(q, k, v, do, True)
     finally:
         flash_mod.DS_WORKSPACE_LIMIT_MIB = saved
-    for a, b in zip(stored, recomputed):
-        assert torch.equal(a, b)
+    for name, a, b in zip(("o", "dq", "dk", "dv"), stored, recomputed):
+        if name == "dq":
+            assert (a.float() - b.float()).abs().max() <= 2e-2 * b.float().abs().max() + 1e-6
+        else:
+            assert torch.equal(a, b), name
     hs = slice(30, 32)
     qs, ks, vs = (t[:, hs].detach().requires_grad_() for t in (q, k, v))
     o_ref = oracle_flash(qs, ks, vs, True, upcast=True)
