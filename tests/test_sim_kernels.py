@@ -87,6 +87,8 @@ DS_CASES = [
     (1, 2, 2, 130, 70, 64, True, torch.float16, True),      # M > N: rows without keys
     (2, 1, 1, 70, 200, 32, False, torch.bfloat16, True),
     (1, 1, 1, 257, 129, 16, True, torch.float16, False),    # three query blocks, key tail of one
+    (1, 1, 1, 270, 200, 128, False, torch.bfloat16, False), # head 128: four whole query tiles and a tail (slotted body)
+    (1, 2, 1, 200, 260, 128, True, torch.float16, True),    # head 128, causal, grouped heads
 ]
 
 
