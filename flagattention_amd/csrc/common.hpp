@@ -6,6 +6,9 @@
 //   * one wavefront multiplies 32x32 blocks with mfma32 (hw.hpp); its lane l owns column l % 32 of a
 //     block and the half h = l / 32 selects which rows / which 8 of the 16 contraction indices.
 #pragma once
+#include <type_traits>
+#include <utility>
+
 #include "hw.hpp"
 
 namespace fa {
@@ -45,6 +48,7 @@ struct TileMover {
   uint32_t stride_bytes, col_bytes;
   int row0, col0;
   int valid;  // rows of the fetched tile that exist
+  uint32_t last_off;
 
   FA_DEVICE void init(int tid, int64_t row_stride) {
     row0 = tid / CPR;
@@ -55,15 +59,27 @@ struct TileMover {
 #pragma unroll
     for (int i = 0; i < PASSES; ++i) goff[i] = (uint32_t)(row0 + i * RPP) * stride_bytes + col_bytes;
   }
-  // rows_valid >= 1 rows of the tile exist
+  // rows_valid >= 1 rows of the tile exist; rows past them load a copy of the last one
   FA_DEVICE void fetch(const T* tile_base, int rows_valid) {
-    valid = rows_valid < ROWS ? rows_valid : ROWS;
-    const uint32_t last = (uint32_t)(valid - 1) * stride_bytes + col_bytes;
+    fetch_begin(rows_valid);
 #pragma unroll
-    for (int i = 0; i < PASSES; ++i) {
-      const uint32_t off = (row0 + i * RPP < valid) ? goff[i] : last;
-      r[i] = *(const u32x4*)((const char*)tile_base + off);
-    }
+    for (int i = 0; i < PASSES; ++i) fetch_pass(tile_base, i);
+  }
+  // the same in pieces, for callers that place the loads themselves
+  FA_DEVICE void fetch_begin(int rows_valid) {
+    valid = rows_valid < ROWS ? rows_valid : ROWS;
+    last_off = (uint32_t)(valid - 1) * stride_bytes + col_bytes;
+  }
+  FA_DEVICE void fetch_pass(const T* tile_base, int i) {
+    const uint32_t off = (row0 + i * RPP < valid) ? goff[i] : last_off;
+    r[i] = *(const u32x4*)((const char*)tile_base + off);
+  }
+  // one pass of commit(), without the zeroes for rows past the end: those keep the copies of the
+  // last row that fetch() loaded
+  template <int LD>
+  FA_DEVICE void commit_pass(T* lds_tile, int i) const {
+    static_assert(kExact, "whole passes only");
+    *(u32x4*)(lds_tile + (row0 + i * RPP) * LD + col0) = r[i];
   }
   template <int LD>
   FA_DEVICE void commit(T* lds_tile) {
@@ -84,6 +100,17 @@ struct TileMover {
 // ---------------------------------------------------------------------------------------------
 // Operand whose contraction index runs along D: element (row = row0 + l % 32, k = k0 + 8h + 0..7)
 // of a row-major tile, one 16-byte LDS read.
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>), in order: a loop whose index is a
+// constant expression inside the body
+template <int... I, class F>
+FA_DEVICE void static_for_each(std::integer_sequence<int, I...>, F&& f) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+FA_DEVICE void static_for(F&& f) {
+  static_for_each(std::make_integer_sequence<int, N>{}, f);
+}
+
 template <class T, int LD>
 FA_DEVICE typename hw::Elem<T>::v8 operand_rowmajor(const T* lds_tile, int row0, int k0, int lane) {
   const T* p = lds_tile + (row0 + (lane & 31)) * LD + k0 + 8 * (lane >> 5);

@@ -80,7 +80,10 @@ struct KvCfg {
   // one wavefront per SIMD: overlap of matrix and element-wise work has to come from the instruction order
   static constexpr bool SLOTTED = WAVES_PER_SIMD == 1 && BM == 64 && D == 128;
   static constexpr size_t STAGE_BYTES = 2 * TILE * sizeof(T) + 2 * BM * sizeof(float);  // Q, dO, L, delta
-  static constexpr size_t LDS_BYTES = 2 * STAGE_BYTES;
+  // the slot-structured body writes the next tile into LDS and passes the barrier before its last
+  // matrix instructions, which still read the current tile: three stages
+  static constexpr int STAGES = SLOTTED ? 3 : 2;
+  static constexpr size_t LDS_BYTES = STAGES * STAGE_BYTES;
 };
 
 // PW (piecewise): the score of (m, n) comes from (q2, k2) when the distance m + pseq - n is >= w and
@@ -168,16 +171,19 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
   // dS = P (dO.v - delta) take one multiplication each in the slots.
   constexpr bool FOLDED = C::SLOTTED && !PW && !DROP;
   const float inv_scale = 1.f / p.sm_scale;
+  auto fetch_stats = [&](int m0) {
+    l_row = m0 + (tid & (C::BM - 1));
+    const int mc = imin(l_row, M - 1);
+    l_reg = lse[mc];
+    d_reg = dlt[mc];
+  };
   auto fetch = [&](int m0) {
     const int rows = M - m0;
     qr.fetch(q_src + (int64_t)m0 * q_stride, rows);
     gr.fetch(gb + (int64_t)m0 * p.dout.st, rows);
     // L and delta of row m0 + tid (threads 0..63), read branch-free from a clamped row and fixed up
     // at commit: nothing may consume a load here, or the wait would cover the tile loads as well
-    l_row = m0 + (tid & (C::BM - 1));
-    const int mc = imin(l_row, M - 1);
-    l_reg = lse[mc];
-    d_reg = dlt[mc];
+    fetch_stats(m0);
   };
   auto commit = [&](int stage) {
     unsigned char* base = smem + stage * C::STAGE_BYTES;
@@ -255,17 +261,21 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
       hw::block_sync();
     }
     hw::wait_global_loads();  // K and V rows
+    // the tile loop starts with the rows of the second tile on their way to registers: every tile
+    // commits its successor to LDS and then requests the tile after that
+    if (t_begin + 1 < t_end) fetch((t_begin + 1) * C::BM);
 
     for (int it = t_begin; it < t_end; ++it) {
       const int m0 = it * C::BM;
       const bool more = it + 1 < t_end;
-      if (more) fetch(m0 + C::BM);
 
       const unsigned char* base = smem + stage * C::STAGE_BYTES;
       const T* sQ = (const T*)base;
       const T* sG = sQ + C::TILE;
       const float* sL = (const float*)(base + 2 * C::TILE * sizeof(T));
       const float* sDl = sL + C::BM;
+      const int next_stage = stage + 1 == C::STAGES ? 0 : stage + 1;
+      bool committed_in_slots = false, synced_in_slots = false, fetched_in_slots = false;
 
       // Tiles that no mask touches (all but the one or two on the diagonal), with one wavefront per
       // SIMD: nothing else would issue under this wavefront's matrix instructions, so the
@@ -280,7 +290,7 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
         constexpr int NA = 2 * C::KSTEPS;       // matrix instructions of an A phase (16)
         constexpr int NC = 4 * (C::DV / 32);    // of a C phase (16)
         static_assert(NA == 16 && NC == 16, "one element of a block per matrix instruction");
-        f32x16 sx[2], dpx[2], prx[2], dsx[2];
+        f32x16 sx[2], dpx[2];
         // operand of A-phase instruction j of block sb, and of C-phase instruction j
         auto a_operand = [&](int sb, int j) {
           return operand_rowmajor<T, C::LD>(j < C::KSTEPS ? sQ : sG, sb * 32, 16 * (j % C::KSTEPS), lane);
@@ -292,82 +302,114 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
           if (j < C::KSTEPS) sx[sb] = hw::mfma32(op, kreg[j], sx[sb]);
           else dpx[sb] = hw::mfma32(op, vreg[j - C::KSTEPS], dpx[sb]);
         };
-        hw::f32x4 lrow[4], drow[4];
-        auto load_rows_stats = [&](int sb) {
+        // the tile's 64 matrix instructions in issue order: A0 (0-15), A1 (16-31), C0 (32-47), C1 (48-63)
+        constexpr int kSlots = 2 * NA + 2 * NC;
+        auto operand = [&](int k) {
+          if (k < NA) return a_operand(0, k);
+          if (k < 2 * NA) return a_operand(1, k - NA);
+          if (k < 2 * NA + NC) return c_operand(0, k - 2 * NA);
+          return c_operand(1, k - 2 * NA - NC);
+        };
+        // accumulators start from the per-row values
+        auto start_scores = [&](int sb) {
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
-            lrow[g] = *(const hw::f32x4*)(sL + sb * 32 + 8 * g + 4 * hh);
-            drow[g] = *(const hw::f32x4*)(sDl + sb * 32 + 8 * g + 4 * hh);
+            const hw::f32x4 l4 = *(const hw::f32x4*)(sL + sb * 32 + 8 * g + 4 * hh);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) sx[sb][4 * g + e] = l4[e];
           }
         };
-        auto element = [&](int sb, int r) {
-          const float pv = hw::exp2_fast(sx[sb][r] * c2);
-          prx[sb][r] = pv;
-          dsx[sb][r] = pv * dpx[sb][r];
+        auto start_dp = [&](int sb) {
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const hw::f32x4 d4 = *(const hw::f32x4*)(sDl + sb * 32 + 8 * g + 4 * hh);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) dpx[sb][4 * g + e] = d4[e];
+          }
         };
-        auto start_block = [&](int sb) {   // accumulators start from the per-row values
-          load_rows_stats(sb);
-#pragma unroll
-          for (int r = 0; r < 16; ++r) { sx[sb][r] = lrow[r >> 2][r & 3]; dpx[sb][r] = drow[r >> 2][r & 3]; }
+        // element r of block sb in two steps one slot apart (the product with dP waits neither for the
+        // exponential nor for the last matrix instruction of the dP chain); a finished pair is packed
+        // at once
+        V8 pa[2][2], da[2][2];
+        float pr_cur = 0.f, pr_prev = 0.f, ds_prev = 0.f;
+        auto elem_p = [&](int sb, int r) {
+          pr_prev = pr_cur;
+          pr_cur = hw::exp2_fast(sx[sb][r] * c2);
+          if (r & 1) { pa[sb][r >> 3][(r & 7) - 1] = (T)pr_prev; pa[sb][r >> 3][r & 7] = (T)pr_cur; }
+        };
+        auto elem_ds = [&](int sb, int r, float pv) {
+          const float dsv = pv * dpx[sb][r];
+          if (r & 1) { da[sb][r >> 3][(r & 7) - 1] = (T)ds_prev; da[sb][r >> 3][r & 7] = (T)dsv; }
+          ds_prev = dsv;
         };
 
-        // ---- A0 ----
-        start_block(0);
-#pragma unroll
-        for (int j = 0; j < NA; ++j) a_issue(0, j, a_operand(0, j));
-        hw::sched_prefetched_operands<NA, 8, 1, 8>();
-        hw::sched_fence();
+        // The next tile's rows (in registers since the previous tile) go to the next stage during the
+        // C1 slots, the workgroup's barrier follows them there, and the loads of the tile after the
+        // next take over the registers one slot after they are free: nothing but the loop edge stands
+        // between this tile's last matrix instruction and the next tile's first.  All of it is
+        // unconditional, because a branch would end the basic block whose order the fences keep: past
+        // the last tile the writes store stale registers into a stage that nobody reads before its
+        // next commit, and the loads fetch the last tile once more.  Rows past M hold copies of row
+        // M - 1 instead of commit()'s zeroes: their P and dS are exact zeroes (L = +inf), and row M - 1
+        // itself is in the same products.
+        constexpr int kPasses = TileMover<T, C::BM, D>::PASSES;
+        constexpr int kCommitSlot = 2 * NA + NC, kSyncSlot = kCommitSlot + 2 * kPasses + 1;
+        constexpr int kFetchSlot = kCommitSlot + kPasses;   // Q registers are free from here on
+        static_assert(TileMover<T, C::BM, D>::kExact && kFetchSlot + 2 * kPasses < kSlots, "fits the C1 slots");
+        const int m_ahead = imin(it + 2, t_end - 1) * C::BM;
+        const T* q_ahead = q_src + (int64_t)m_ahead * q_stride;
+        const T* g_ahead = gb + (int64_t)m_ahead * p.dout.st;
+        committed_in_slots = synced_in_slots = fetched_in_slots = true;
+        T* nQ = (T*)(smem + next_stage * C::STAGE_BYTES);
+        T* nG = nQ + C::TILE;
+        float* nf = (float*)(nG + C::TILE);
 
-        // ---- A1 with E0 ----
-        constexpr int kDepthA = 4;
-        V8 ring_a[kDepthA];
-        start_block(1);
+        constexpr int kDepth = 4;
+        V8 ring[kDepth];
+        start_scores(0);
 #pragma unroll
-        for (int j = 0; j < kDepthA; ++j) ring_a[j] = a_operand(1, j);
+        for (int k = 0; k < kDepth; ++k) ring[k] = operand(k);
+        start_dp(0);
         hw::sched_fence();
-#pragma unroll
-        for (int j = 0; j < NA; ++j) {
-          a_issue(1, j, ring_a[j % kDepthA]);
-          if (j + kDepthA < NA) ring_a[j % kDepthA] = a_operand(1, j + kDepthA);
-          element(0, j);
+        static_for<kSlots>([&](auto slot) {
+          constexpr int k = decltype(slot)::value;
+          const V8 op = ring[k % kDepth];
+          if constexpr (k < 2 * NA) {
+            a_issue(k / NA, k % NA, op);
+          } else {
+            constexpr int sb = (k - 2 * NA) / NC, j = (k - 2 * NA) % NC, c = j >> 3, db = j & 3;
+            if constexpr ((j & 4) != 0) dk[db] = hw::mfma32(da[sb][c], op, dk[db]);
+            else dv[db] = hw::mfma32(pa[sb][c], op, dv[db]);
+            if (DS && (j & 7) == 0)
+              hw::store_streaming(ds_row + (int64_t)(m0 / 32 + sb) * 1024 + c * 512,
+                                  __builtin_bit_cast(u32x4, da[sb][c]));
+          }
+          if constexpr (k + kDepth < kSlots) ring[k % kDepth] = operand(k + kDepth);
+          if constexpr (k == NA - 6) start_scores(1);
+          if constexpr (k == NA + 2) start_dp(1);
+          // E0 under A1, E1 under C0; the last product of a block under the next phase's first slot
+          if constexpr (k >= NA && k < NA + 32) {
+            constexpr int e = k - NA, sb = e >> 4, r = e & 15;
+            if constexpr (e > 0) elem_ds((e - 1) >> 4, (e - 1) & 15, pr_cur);
+            elem_p(sb, r);
+          }
+          if constexpr (k == NA + 32) elem_ds(1, 15, pr_cur);
+          if constexpr (k >= kCommitSlot && k < kCommitSlot + kPasses)
+            qr.template commit_pass<C::LD>(nQ, k - kCommitSlot);
+          if constexpr (k >= kCommitSlot + kPasses && k < kCommitSlot + 2 * kPasses)
+            gr.template commit_pass<C::LD>(nG, k - kCommitSlot - kPasses);
+          if constexpr (k == kCommitSlot + 2 * kPasses) {  // every wavefront writes the same 64 + 64 values
+            nf[tid & (C::BM - 1)] = l_row < M ? -l_reg * inv_scale : -__builtin_inff();
+            nf[C::BM + (tid & (C::BM - 1))] = l_row < M ? -d_reg : 0.f;
+          }
+          if constexpr (k == kSyncSlot) hw::block_sync();
+          if constexpr (k == kFetchSlot) { qr.fetch_begin(M - m_ahead); gr.fetch_begin(M - m_ahead); }
+          if constexpr (k >= kFetchSlot && k < kFetchSlot + kPasses) qr.fetch_pass(q_ahead, k - kFetchSlot);
+          if constexpr (k >= kFetchSlot + kPasses && k < kFetchSlot + 2 * kPasses)
+            gr.fetch_pass(g_ahead, k - kFetchSlot - kPasses);
+          if constexpr (k == kFetchSlot + 2 * kPasses) fetch_stats(m_ahead);
           hw::sched_fence();
-        }
-
-        // ---- C0 with E1 ----
-        constexpr int kDepthC = 3;
-        V8 ring_c[kDepthC];
-        V8 pa[2], da[2];
-#pragma unroll
-        for (int c = 0; c < 2; ++c) { pa[c] = pack_half_block<T>(prx[0], c); da[c] = pack_half_block<T>(dsx[0], c); }
-#pragma unroll
-        for (int j = 0; j < kDepthC; ++j) ring_c[j] = c_operand(0, j);
-        hw::sched_fence();
-#pragma unroll
-        for (int j = 0; j < NC; ++j) {
-          const int c = j >> 3, db = j & 3;
-          if (j & 4) dk[db] = hw::mfma32(da[c], ring_c[j % kDepthC], dk[db]);
-          else dv[db] = hw::mfma32(pa[c], ring_c[j % kDepthC], dv[db]);
-          if (j + kDepthC < NC) ring_c[j % kDepthC] = c_operand(0, j + kDepthC);
-          if (DS && (j & 7) == 0)
-            hw::store_streaming(ds_row + (int64_t)(m0 / 32) * 1024 + c * 512, __builtin_bit_cast(u32x4, da[c]));
-          element(1, j);
-          hw::sched_fence();
-        }
-
-        // ---- C1 ----
-#pragma unroll
-        for (int c = 0; c < 2; ++c) {
-          V8 pa1 = pack_half_block<T>(prx[1], c);
-#pragma unroll
-          for (int db = 0; db < C::DV / 32; ++db)
-            dv[db] = hw::mfma32(pa1, operand_transposed<T, C::LD>(sG, 32 + 16 * c, db * 32, lane), dv[db]);
-          V8 da1 = pack_half_block<T>(dsx[1], c);
-          if (DS) hw::store_streaming(ds_row + (int64_t)(m0 / 32 + 1) * 1024 + c * 512, __builtin_bit_cast(u32x4, da1));
-#pragma unroll
-          for (int db = 0; db < C::DV / 32; ++db)
-            dk[db] = hw::mfma32(da1, operand_transposed<T, C::LD>(sQ, 32 + 16 * c, db * 32, lane), dk[db]);
-        }
-        hw::sched_prefetched_operands<NC, 5, 2>();
+        });
       }
       }
       if (!plain_tile) {
@@ -448,9 +490,10 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
       }
       }
 
-      if (more) commit(stage ^ 1);
-      hw::block_sync();
-      stage ^= 1;
+      if (more && !committed_in_slots) commit(next_stage);
+      if (!synced_in_slots) hw::block_sync();
+      if (!fetched_in_slots && it + 2 < t_end) fetch(m0 + 2 * C::BM);
+      stage = next_stage;
     }
 
     if (PW) {  // this regime's dK is complete (piecewise has no grouped heads)
