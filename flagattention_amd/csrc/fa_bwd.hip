@@ -169,7 +169,7 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
   // In the instantiation with the slot-structured body, LDS holds -L / sm_scale and -delta per row:
   // the score and dP accumulators start from them, so that P = exp2(c2 (q.k - L / sm_scale)) and
   // dS = P (dO.v - delta) take one multiplication each in the slots.
-  constexpr bool FOLDED = C::SLOTTED && !PW && !DROP;
+  constexpr bool FOLDED = C::SLOTTED && !DROP;
   const float inv_scale = 1.f / p.sm_scale;
   auto fetch_stats = [&](int m0) {
     l_row = m0 + (tid & (C::BM - 1));
@@ -284,8 +284,12 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
       //   A0 | A1 with E0 | C0 with E1 | C1      (A: S and dP, E: P and dS, C: dV and dK)
       // and a scheduling fence after every such slot keeps the compiler from regrouping them.
       bool plain_tile = false;
-      if constexpr (C::SLOTTED && !PW && !DROP) plain_tile = !p.causal || (m0 + pseq >= nw + 31);
-      if constexpr (C::SLOTTED && !PW && !DROP) {
+      if constexpr (FOLDED) {
+        plain_tile = !p.causal || (m0 + pseq >= nw + 31);
+        // piecewise: every entry of the 64 x 32 tile belongs to this pass's regime
+        if (PW) plain_tile = plain_tile && (far_phase ? (m0 + pseq - (nw + 31) >= p.w) : (m0 + 63 + pseq - nw < p.w));
+      }
+      if constexpr (FOLDED) {
       if (plain_tile) {
         constexpr int NA = 2 * C::KSTEPS;       // matrix instructions of an A phase (16)
         constexpr int NC = 4 * (C::DV / 32);    // of a C phase (16)
