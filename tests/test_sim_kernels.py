@@ -215,6 +215,7 @@ PW_CASES = [
     (1, 1, 70, 330, 32, -1000, False, torch.bfloat16),  # non-causal, every pair far
     (1, 1, 330, 70, 32, 129, False, torch.float16),     # M > N, threshold on a block edge
     (2, 2, 200, 330, 128, 64, True, torch.bfloat16),    # head size 128, threshold on a block edge, two heads
+    (1, 1, 270, 300, 128, 200, False, torch.bfloat16),  # head size 128: whole tiles in the near regime, and in the far one
 ]
 
 
