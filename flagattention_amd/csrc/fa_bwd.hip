@@ -331,21 +331,23 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
             for (int e = 0; e < 4; ++e) dpx[sb][4 * g + e] = d4[e];
           }
         };
-        // element r of block sb in two steps one slot apart (the product with dP waits neither for the
-        // exponential nor for the last matrix instruction of the dP chain); a finished pair is packed
-        // at once
+        // element r of a block in two steps, each as early as its inputs exist, so that the element-wise
+        // work spreads over as many slots as the data dependencies allow: p = exp2(c s) of block 0 from
+        // the slot after its S chain ended (kP0), dS = p dP eight slots behind it, block 1 likewise a
+        // phase later; a finished pair is packed at once
         V8 pa[2][2], da[2][2];
-        float pr_cur = 0.f, pr_prev = 0.f, ds_prev = 0.f;
+        float pr[2][16];
+        float ds_prev = 0.f;
         auto elem_p = [&](int sb, int r) {
-          pr_prev = pr_cur;
-          pr_cur = hw::exp2_fast(sx[sb][r] * c2);
-          if (r & 1) { pa[sb][r >> 3][(r & 7) - 1] = (T)pr_prev; pa[sb][r >> 3][r & 7] = (T)pr_cur; }
+          pr[sb][r] = hw::exp2_fast(sx[sb][r] * c2);
+          if (r & 1) { pa[sb][r >> 3][(r & 7) - 1] = (T)pr[sb][r - 1]; pa[sb][r >> 3][r & 7] = (T)pr[sb][r]; }
         };
-        auto elem_ds = [&](int sb, int r, float pv) {
-          const float dsv = pv * dpx[sb][r];
+        auto elem_ds = [&](int sb, int r) {
+          const float dsv = pr[sb][r] * dpx[sb][r];
           if (r & 1) { da[sb][r >> 3][(r & 7) - 1] = (T)ds_prev; da[sb][r >> 3][r & 7] = (T)dsv; }
           ds_prev = dsv;
         };
+        constexpr int kP0 = C::KSTEPS + 1, kD0 = NA + 1, kP1 = NA + C::KSTEPS + 1, kD1 = 2 * NA + 1;
 
         // The next tile's rows (in registers since the previous tile) go to the next stage during the
         // C1 slots, the workgroup's barrier follows them there, and the loads of the tile after the
@@ -391,13 +393,10 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
           if constexpr (k + kDepth < kSlots) ring[k % kDepth] = operand(k + kDepth);
           if constexpr (k == NA - 6) start_scores(1);
           if constexpr (k == NA + 2) start_dp(1);
-          // E0 under A1, E1 under C0; the last product of a block under the next phase's first slot
-          if constexpr (k >= NA && k < NA + 32) {
-            constexpr int e = k - NA, sb = e >> 4, r = e & 15;
-            if constexpr (e > 0) elem_ds((e - 1) >> 4, (e - 1) & 15, pr_cur);
-            elem_p(sb, r);
-          }
-          if constexpr (k == NA + 32) elem_ds(1, 15, pr_cur);
+          if constexpr (k >= kD0 && k < kD0 + 16) elem_ds(0, k - kD0);
+          if constexpr (k >= kD1 && k < kD1 + 16) elem_ds(1, k - kD1);
+          if constexpr (k >= kP0 && k < kP0 + 16) elem_p(0, k - kP0);
+          if constexpr (k >= kP1 && k < kP1 + 16) elem_p(1, k - kP1);
           if constexpr (k >= kCommitSlot && k < kCommitSlot + kPasses)
             qr.template commit_pass<C::LD>(nQ, k - kCommitSlot);
           if constexpr (k >= kCommitSlot + kPasses && k < kCommitSlot + 2 * kPasses)
