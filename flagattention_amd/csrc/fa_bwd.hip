@@ -261,6 +261,10 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
       hw::block_sync();
     }
     hw::wait_global_loads();  // K and V rows
+    if constexpr (FOLDED) {
+#pragma unroll
+      for (int kk = 0; kk < C::KSTEPS; ++kk) { hw::keep_in_agprs(kreg[kk]); hw::keep_in_agprs(vreg[kk]); }
+    }
     // the tile loop starts with the rows of the second tile on their way to registers: every tile
     // commits its successor to LDS and then requests the tile after that
     if (t_begin + 1 < t_end) fetch((t_begin + 1) * C::BM);
@@ -303,8 +307,8 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
           return operand_transposed<T, C::LD>((j & 4) ? sQ : sG, sb * 32 + 16 * (j >> 3), (j & 3) * 32, lane);
         };
         auto a_issue = [&](int sb, int j, const V8& op) {
-          if (j < C::KSTEPS) sx[sb] = hw::mfma32(op, kreg[j], sx[sb]);
-          else dpx[sb] = hw::mfma32(op, vreg[j - C::KSTEPS], dpx[sb]);
+          if (j < C::KSTEPS) sx[sb] = hw::mfma32_vacc(op, kreg[j], sx[sb]);
+          else dpx[sb] = hw::mfma32_vacc(op, vreg[j - C::KSTEPS], dpx[sb]);
         };
         // the tile's 64 matrix instructions in issue order: A0 (0-15), A1 (16-31), C0 (32-47), C1 (48-63)
         constexpr int kSlots = 2 * NA + 2 * NC;

@@ -60,6 +60,23 @@ FA_DEVICE f32x16 mfma32(half8 a, half8 b, f32x16 c) {
 FA_DEVICE f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
 }
+// The same product with the accumulator pinned to VGPRs and the B operand to AGPRs.  Left to itself
+// the compiler keeps every accumulator of a kernel that may use all 512 registers in AGPRs, from where
+// each element costs a v_accvgpr_read before the vector ALU can touch it; here the accumulator is what
+// the vector ALU works on and the B operand (a register-resident K or V row) is what can live in AGPRs.
+// The compiler does not see into the assembly, so the CALLER keeps the distance the hardware needs
+// between this instruction and a vector-ALU read of its result: another matrix instruction in between.
+FA_DEVICE f32x16 mfma32_vacc(half8 a, half8 b, f32x16 c) {
+  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
+  return c;
+}
+FA_DEVICE f32x16 mfma32_vacc(bf16x8 a, bf16x8 b, f32x16 c) {
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
+  return c;
+}
+// Moves a register-resident operand to AGPRs for good (what mfma32_vacc takes as B).
+template <class V>
+FA_DEVICE void keep_in_agprs(V& v) { asm volatile("" : "+a"(v)); }
 // D(16x16) += A(16x32) * B(32x16).  Lane l holds, for q = l / 16:
 //   A[i = l % 16][k = 8q + e]     B[k = 8q + e][j = l % 16]     D[i = 4q + r][j = l % 16], r = 0..3
 FA_DEVICE f32x4 mfma16(half8 a, half8 b, f32x4 c) {

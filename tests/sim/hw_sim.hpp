@@ -216,6 +216,8 @@ template <class V8> inline f32x16 mfma32_any(V8 a, V8 b, f32x16 c) {
 }
 inline f32x16 mfma32(half8 a, half8 b, f32x16 c) { return mfma32_any(a, b, c); }
 inline f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) { return mfma32_any(a, b, c); }
+inline f32x16 mfma32_vacc(half8 a, half8 b, f32x16 c) { return mfma32_any(a, b, c); }
+inline f32x16 mfma32_vacc(bf16x8 a, bf16x8 b, f32x16 c) { return mfma32_any(a, b, c); }
 
 template <class V8> inline f32x4 mfma16_any(V8 a, V8 b, f32x4 c) {
   hwsim::Lane& ln = hwsim::lanes[hwsim::cur];
@@ -257,6 +259,7 @@ inline bool wave_any(bool pred) {
 }
 
 inline void sched_fence() {}
+template <class V> inline void keep_in_agprs(V&) {}
 inline void keep_branch() {}
 template <int N, int DEPTH, int RPM = 1, int EXTRA = 0> inline void sched_prefetched_operands() {}
 inline float exp2_fast(float x) { return exp2f(x); }
