@@ -289,7 +289,9 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
       // and a scheduling fence after every such slot keeps the compiler from regrouping them.
       bool plain_tile = false;
       if constexpr (FOLDED) {
-        plain_tile = !p.causal || (m0 + pseq >= nw + 31);
+        // a block with keys past N goes through the masked path: its P and dS must be exact zeroes
+        // there (K and V rows are zero, so the score is just -L and exp2 of it can be huge)
+        plain_tile = (nw + 31 < N) && (!p.causal || (m0 + pseq >= nw + 31));
         // piecewise: every entry of the 64 x 32 tile belongs to this pass's regime
         if (PW) plain_tile = plain_tile && (far_phase ? (m0 + pseq - (nw + 31) >= p.w) : (m0 + 63 + pseq - nw < p.w));
       }
@@ -437,7 +439,7 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
           dp = hw::mfma32(operand_rowmajor<T, C::LD>(sG, sb * 32, 16 * kk, lane), vreg[kk], dp);
         hw::sched_prefetched_operands<2 * C::KSTEPS, (C::KSTEPS >= 8 ? 8 : 2)>();
 
-        bool need_mask = p.causal && (mr0 + pseq < nw + 31);
+        bool need_mask = (nw + 31 >= N) || (p.causal && (mr0 + pseq < nw + 31));
         if (PW) need_mask = need_mask || (far_phase ? (mr0 + pseq - (nw + 31) < p.w) : (mr0 + 31 + pseq - nw >= p.w));
         // L * log2e and delta of this lane's 16 query rows: rows 8g + 4h + 0..3 are contiguous
         hw::f32x4 lrow[4], drow[4];
@@ -451,7 +453,7 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
             const int m = mr0 + block_row(r, hh);
-            bool keep = !p.causal || (m + pseq >= my_n);
+            bool keep = (my_n < N) && (!p.causal || (m + pseq >= my_n));
             if (PW) keep = keep && ((m + pseq - my_n >= p.w) == far_phase);
             float pv = FOLDED ? hw::exp2_fast((s[r] + lrow[r >> 2][r & 3]) * c2)
                               : hw::exp2_fast(fmaf(s[r], c2, -lrow[r >> 2][r & 3]));

@@ -48,3 +48,39 @@ def test_missing_library_raises(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
     with pytest.raises(RuntimeError, match="no fallback"):
         _lib.get()
+
+
+def test_integration_doc_binding_matches_signature_table():
+    """The worked ctypes binding in the integration document is evaluated as written (with a stand-in
+    for the loaded library) and its argument types must equal the loader's table for fa_fwd."""
+    import ctypes
+    import types
+    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    blocks = re.findall(r"```python\n(.*?)```", text, flags=re.S)
+    block = next(b for b in blocks if "fa_fwd.argtypes" in b)
+    # everything up to the helper that touches tensors: struct, library handle, argtypes, restype
+    setup = block.split("def _view")[0]
+    setup = setup.replace("import ctypes, torch", "import ctypes")
+    fake_lib = types.SimpleNamespace(fa_fwd=types.SimpleNamespace())
+    setup = setup.replace('ctypes.CDLL("libflagattn_hip.so")', "_fake_lib")
+    env = {"_fake_lib": fake_lib}
+    exec(setup, env)
+    doc_types = fake_lib.fa_fwd.argtypes
+    table = _lib.SIGNATURES["fa_fwd"]
+    assert len(doc_types) == len(table) == declared_functions()["fa_fwd"]
+    for i, (d, t) in enumerate(zip(doc_types, table)):
+        if t is _lib._v:   # pointer to the view struct: the document declares its own mirror of it
+            assert issubclass(d, ctypes._Pointer) and \
+                [f[0] for f in d._type_._fields_] == [f[0] for f in _lib.View4._fields_], i
+        else:
+            assert d is t, (i, d, t)
+    assert fake_lib.fa_fwd.restype is ctypes.c_int
+    # the call in the document passes as many arguments as the binding declares
+    call = re.search(r"_lib\.fa_fwd\((.*?)\)\nassert rc == 0", block, flags=re.S).group(1)
+    call = re.sub(r"#.*", "", call)
+    depth, nargs = 0, 1
+    for ch in call:
+        depth += ch in "([" 
+        depth -= ch in ")]"
+        nargs += (ch == "," and depth == 0)
+    assert nargs == len(table)

@@ -312,3 +312,34 @@ def test_dropout_advances_the_generator_and_is_reproducible():
     with pytest.raises(AssertionError):   # decode shapes take the split-KV path, which has no dropout
         flag_attn.flash_attention(q[:1, :2, :1], make((1, 2, 8192, 64), torch.float16, "BHTD", 1.0, 5),
                                   make((1, 2, 8192, 64), torch.float16, "BHTD", 1.0, 6), dropout_p=0.5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("M,N", [(1024, 1000), (2048, 1031), (1024, 2049)])
+def test_ds_route_with_key_tail_and_very_negative_log_normalizer(M, N, causal, dtype):
+    """Head size 128 at M * N >= 2^20 takes the route that keeps dS.  With a key count that is no
+    multiple of 32 and log-normalizers below -11.5, exp(-L) of the lanes past the last key overflows
+    fp16: those dS entries must be exact zeroes, or dQ becomes NaN.  dQ of the public backward is
+    compared with the recomputing dQ kernel (same products, same rounding of dS) and with the oracle."""
+    from flagattention_amd import _abi, _lib
+    lib = _lib.get()
+    g = torch.Generator(device="cuda").manual_seed(7)
+    D = 128
+    q = (torch.randn(1, 2, M, D, device="cuda", generator=g) * 0.1 + 1.0).to(dtype).requires_grad_()
+    k = (torch.randn(1, 2, N, D, device="cuda", generator=g) * 0.1 - 2.0).to(dtype).requires_grad_()
+    v = torch.randn(1, 2, N, D, device="cuda", generator=g).to(dtype).requires_grad_()
+    do = torch.randn(1, 2, M, D, device="cuda", generator=g).to(dtype)
+    o, lse, *_ = flag_attn.flash_attention(q, k, v, causal, return_log_normalizer=True)
+    assert lse[torch.isfinite(lse)].max() < -11.5
+    dq, dk, dv = torch.autograd.grad(o, (q, k, v), do)
+    assert torch.isfinite(dq.float()).all() and torch.isfinite(dk.float()).all()
+    delta = torch.empty_like(lse)
+    _abi.fa_bwd_delta(lib, o.detach(), do, delta)
+    dq_plain = torch.empty_like(dq)
+    _abi.fa_bwd_dq(lib, q.detach(), k.detach(), v.detach(), do, lse, delta, dq_plain, causal, D ** -0.5)
+    assert (dq.float() - dq_plain.float()).abs().max() <= 2e-2 * dq_plain.float().abs().max() + 1e-6
+    ref = torch.autograd.grad(oracle_flash(q, k, v, causal, upcast=True), (q, k, v), do)
+    same = torch.autograd.grad(oracle_flash(q, k, v, causal, upcast=False), (q, k, v), do)
+    for name, h, s, r in zip(("dq", "dk", "dv"), (dq, dk, dv), same, ref):
+        check(name, h, s, r)

@@ -132,6 +132,34 @@ def test_flash_backward_with_stored_ds(lib, B, H, Hk, M, N, D, causal, dtype, bt
     assert (dq.float() - dq_plain.float()).abs().max() <= 2e-2 * dq_plain.float().abs().max() + 1e-6
 
 
+@pytest.mark.parametrize("dtype,causal,M,N", [
+    (torch.float16, False, 64, 40), (torch.float16, False, 128, 200), (torch.float16, True, 100, 170),
+    (torch.bfloat16, False, 64, 40)])
+def test_stored_ds_is_zero_for_keys_past_the_end(lib, dtype, causal, M, N):
+    """Head size 128, a key count that is no multiple of 32 and strongly negative log-normalizers: the
+    lanes of keys past N see zero K/V rows, so exp2(score - L) there is exp(-L), far above fp16's range
+    once rounded.  The dK/dV kernel must leave exact zeroes for them in the dS workspace, or the
+    dQ-from-dS kernel multiplies infinities by its zeroed K rows."""
+    D, sc = 128, 128 ** -0.5
+    q = (torch.randn(1, 1, M, D) * 0.1 + 1.0).to(dtype)
+    k = (torch.randn(1, 1, N, D) * 0.1 - 1.8).to(dtype)
+    v = torch.randn(1, 1, N, D).to(dtype)
+    do = torch.randn(1, 1, M, D).to(dtype)
+    o = torch.empty_like(q)
+    lse = torch.empty(1, 1, M)
+    _abi.fa_fwd(lib, q, k, v, o, lse, causal, sc)
+    assert lse.max() < -11.5   # exp(-L) does not fit fp16
+    delta = torch.empty(1, 1, M)
+    _abi.fa_bwd_delta(lib, o, do, delta)
+    dk, dv, dq, dq_plain = (torch.empty_like(t) for t in (k, v, q, q))
+    ds = torch.full((lib.fa_bwd_ds_workspace_mib(1, 1, M, N) << 19,), float("nan"), dtype=dtype)
+    _abi.fa_bwd_dkdv_ds(lib, q, k, v, do, lse, delta, dk, dv, ds, causal, sc)
+    _abi.fa_bwd_dq_from_ds(lib, k, ds, dq, causal, sc)
+    _abi.fa_bwd_dq(lib, q, k, v, do, lse, delta, dq_plain, causal, sc)
+    assert torch.isfinite(dq.float()).all()
+    assert (dq.float() - dq_plain.float()).abs().max() <= 2e-2 * dq_plain.float().abs().max() + 1e-6
+
+
 @pytest.mark.parametrize("B,H,M,N,pd,seed,offset", [
     (1, 2, 7, 33, 0.3, 1234, 40),                                   # 462 elements: a vector tail
     (2, 1, 16, 16, 0.5, 987654321987, 123456789123456789),          # 64-bit counter, whole vectors only
