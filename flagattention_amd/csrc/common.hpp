@@ -194,13 +194,6 @@ FA_DEVICE bool dropout_keeps(uint64_t counter, uint64_t seed, float dropout_p) {
 // ---------------------------------------------------------------------------------------------
 // launch
 // ---------------------------------------------------------------------------------------------
-#ifdef FLAGATTN_HOST_SIM
-template <class P>
-int launch(void (*kern)(P), dim3 grid, size_t lds_bytes, hipStream_t, const P& p) {
-  hwsim::run_grid(grid, kThreads, lds_bytes, [&]() { kern(p); });
-  return 0;
-}
-#else
 template <class P>
 int launch(void (*kern)(P), dim3 grid, size_t lds_bytes, hipStream_t stream, const P& p) {
   if (lds_bytes > 48 * 1024) {
@@ -211,7 +204,6 @@ int launch(void (*kern)(P), dim3 grid, size_t lds_bytes, hipStream_t stream, con
   hipLaunchKernelGGL(kern, grid, dim3(kThreads), lds_bytes, stream, p);
   return (int)hipGetLastError();
 }
-#endif
 
 // error codes of the C entry points (positive values are hipError_t)
 constexpr int kOk = 0;

@@ -354,6 +354,31 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
           ds_prev = dsv;
         };
         constexpr int kP0 = C::KSTEPS + 1, kD0 = NA + 1, kP1 = NA + C::KSTEPS + 1, kD1 = 2 * NA + 1;
+        // hw::mfma32_vacc hides its result registers from the compiler's hazard handling, so the slot
+        // order itself has to keep a vector-ALU read of sx / dpx behind the matrix instruction that
+        // wrote them last.  A 32x32x16 product occupies the matrix pipe for 16 passes and its result
+        // may be read 18 cycles' worth of wait states after its last pass; a slot issues its matrix
+        // instruction first and its element-wise work after it.  If the chain's last product sits in
+        // slot w, the product of slot w + 1 cannot issue before w has left the pipe's front and the
+        // product of slot w + 2 cannot issue before w has written back, so element-wise work of slot
+        // r >= w + 2 reads finished registers: one whole other matrix instruction lies in between.
+        constexpr int kLastS0 = C::KSTEPS - 1, kLastDp0 = NA - 1, kLastS1 = NA + C::KSTEPS - 1, kLastDp1 = 2 * NA - 1;
+        constexpr int kHazardSlots = 2;
+        static_assert(kP0 >= kLastS0 + kHazardSlots, "exp2 of block 0 reads S before its last product has written back");
+        static_assert(kD0 >= kLastDp0 + kHazardSlots, "dS of block 0 reads dP before its last product has written back");
+        static_assert(kP1 >= kLastS1 + kHazardSlots, "exp2 of block 1 reads S before its last product has written back");
+        static_assert(kD1 >= kLastDp1 + kHazardSlots, "dS of block 1 reads dP before its last product has written back");
+        static_assert(kD0 >= kP0 && kD1 >= kP1, "dS = p * dP needs p of the same element");
+        // operands are packed in pairs as soon as their second element exists; the dV / dK products that
+        // consume half block c of block sb sit in C-phase slots 8c .. 8c + 3 (dV) and 8c + 4 .. 8c + 7 (dK)
+        static_assert(kP0 + 7 < 2 * NA && kP0 + 15 < 2 * NA + 8, "P of block 0 is packed before dV takes it");
+        static_assert(kD0 + 7 < 2 * NA + 4 && kD0 + 15 < 2 * NA + 12, "dS of block 0 is packed before dK takes it");
+        static_assert(kP1 + 7 < 2 * NA + NC && kP1 + 15 < 2 * NA + NC + 8, "P of block 1 is packed before dV takes it");
+        static_assert(kD1 + 7 < 2 * NA + NC + 4 && kD1 + 15 < 2 * NA + NC + 12, "dS of block 1 is packed before dK takes it");
+        // the accumulators of block 1 are re-initialised (start_scores(1) in slot NA - 6, start_dp(1) in
+        // slot NA + 2) while block 1's own chains have not started and block 0's element-wise work reads
+        // only sx[0] / dpx[0]
+        static_assert(NA - 6 >= 0 && NA + 2 < NA + C::KSTEPS, "block 1 starts from its rows' values before its chains run");
 
         // The next tile's rows (in registers since the previous tile) go to the next stage during the
         // C1 slots, the workgroup's barrier follows them there, and the loads of the tile after the

@@ -57,11 +57,7 @@ struct TotalParams {
 
 }  // namespace fa
 
-#ifdef FLAGATTN_HOST_SIM
-typedef void* hipStream_t;
-#else
-#include <hip/hip_runtime.h>
-#endif
+#include "hw.hpp"  // hipStream_t
 
 namespace fa {
 int run_fwd(const FwdParams& p, bool piecewise, hipStream_t stream);

@@ -10,7 +10,7 @@ import os
 
 import torch
 
-from . import _abi, _lib
+from . import _abi, _config, _lib
 from .split_kv import (num_splits_heuristic, split_kv_forward, SPLIT_BLOCK_M, SPLIT_BLOCK_N,
                        DECODE_MAX_ROWS)
 from .total import _total_attention
@@ -21,17 +21,24 @@ __all__ = ["attention"]
 _HEAD_DIMS = (16, 32, 64, 128)
 
 
-def get_fwd_config(B, H, M, N, D, causal):
-    """(BLOCK_M, BLOCK_N, num_stages, num_warps) of the dense forward kernel.
+# (BLOCK_M, BLOCK_N) the kernels are compiled for; the first entry is the default
+FWD_TILES = ((128, 64),)
+BWD_TILES = ((64, 128),)
 
-    Kept as an overridable module-level hook like ``src/flag_attn/flash.py:290-322``; on gfx950 the
-    tile shape is compiled into the kernel (128 query rows per workgroup, 64-key pipeline stages,
-    two LDS stages, four 64-lane wavefronts), so the value is informational."""
+
+def get_fwd_config(B, H, M, N, D, causal):
+    """(BLOCK_M, BLOCK_N, num_stages, num_warps) of the dense forward kernel: query rows per
+    workgroup, keys per pipeline stage, LDS stages, 64-lane wavefronts.
+
+    An overridable module-level hook like ``src/flag_attn/flash.py:290-322``, called before every
+    forward launch (``flash.py:64-66``).  The kernels are compiled ahead of time, so an override may
+    only choose among ``FWD_TILES``; any other answer is reported once and the default is launched."""
     return (128, 64, 2, 4)
 
 
 def get_bwd_config(B, H, M, N, D, causal):
-    """(BLOCK_M, BLOCK_N, num_stages, num_warps) of the dK/dV kernel (``flash.py:493-519`` hook)."""
+    """(BLOCK_M, BLOCK_N, num_stages, num_warps) of the dK/dV kernel: queries per pipeline step, keys
+    per workgroup (``flash.py:493-519`` hook, called as in ``flash.py:185-186``; see ``BWD_TILES``)."""
     return (64, 128, 2, 4)
 
 
@@ -68,6 +75,8 @@ class FlashAttention(torch.autograd.Function):
             if splits > 1 or (M <= DECODE_MAX_ROWS and N >= 1024 and not is_dropout):
                 o, L = split_kv_forward(lib, q, k, v, causal, sm_scale, splits)
             else:
+                # looked up by name at call time, so that an assignment to flash.get_fwd_config takes effect
+                _config.resolve(get_fwd_config, FWD_TILES, "flash_attention forward", (B, H, M, N, D, causal))
                 o = torch.empty_like(q)
                 if not _abi.is_kernel_ready(o):
                     o = torch.empty(q.shape, dtype=q.dtype, device=q.device)
@@ -100,6 +109,7 @@ class FlashAttention(torch.autograd.Function):
         lib = _lib.get()
         do = _abi.kernel_ready(do)
         with torch.cuda.device(q.device):
+            _config.resolve(get_bwd_config, BWD_TILES, "flash_attention backward", (B, H, M, N, D, causal))
             delta = torch.empty_like(L)
             _abi.fa_bwd_delta(lib, o, do, delta)
             # dK/dV come out summed over each kv head's group of query heads (flash.py:205-206,250-251

@@ -8,18 +8,24 @@ import math
 
 import torch
 
-from . import _abi, _lib
+from . import _abi, _config, _lib
 from .flash import _ds_workspace, ds_heads_per_launch
 
 __all__ = ["attention"]
 
 
+FWD_TILES = ((128, 64),)
+BWD_TILES = ((64, 128),)
+
+
 def get_fwd_config(B, H, M, N, D, causal):
-    """Informational; the tile shape is compiled into the kernel (``piecewise.py:194-221`` hook)."""
+    """(BLOCK_M, BLOCK_N, num_stages, num_warps); overridable hook called before the forward launch
+    (``piecewise.py:44, 194-221``).  Only ``FWD_TILES`` are compiled; another answer is reported once."""
     return (128, 64, 2, 4)
 
 
 def get_bwd_config(B, H, M, N, D, causal):
+    """The same for the dK/dV kernel (``piecewise.py:98-99, 373-405``; ``BWD_TILES``)."""
     return (64, 128, 2, 4)
 
 
@@ -35,6 +41,8 @@ class PiecewiseAttention(torch.autograd.Function):
         lib = _lib.get()
         q1, k1, q2, k2, v = (_abi.kernel_ready(t) for t in (q1, k1, q2, k2, v))
         with torch.cuda.device(q1.device):
+            _config.resolve(get_fwd_config, FWD_TILES, "piecewise_attention forward",
+                            (B, H, M, k1.shape[2], D, causal))
             o = torch.empty_like(q1)
             if not _abi.is_kernel_ready(o):
                 o = torch.empty(q1.shape, dtype=q1.dtype, device=q1.device)
@@ -50,6 +58,8 @@ class PiecewiseAttention(torch.autograd.Function):
         lib = _lib.get()
         do = _abi.kernel_ready(do)
         with torch.cuda.device(q1.device):
+            _config.resolve(get_bwd_config, BWD_TILES, "piecewise_attention backward",
+                            (q1.shape[0], q1.shape[1], q1.shape[2], k1.shape[2], q1.shape[3], ctx.causal))
             delta = torch.empty_like(L)
             _abi.fa_bwd_delta(lib, o, do, delta)
             dk1 = torch.empty(k1.shape, dtype=k1.dtype, device=k1.device)

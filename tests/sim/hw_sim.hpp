@@ -26,6 +26,23 @@ extern "C" void __sanitizer_finish_switch_fiber(void* fake_stack_save, const voi
 typedef void* hipStream_t;
 struct dim3 { unsigned x, y, z; dim3(unsigned a = 1, unsigned b = 1, unsigned c = 1) : x(a), y(b), z(c) {} };
 
+// The few host-side HIP calls the library makes, for a "device" that is this process: one device with
+// 256 compute units, device symbols are ordinary globals, a launch runs the grid to completion.
+typedef int hipError_t;
+constexpr hipError_t hipSuccess = 0;
+enum hipFuncAttribute { hipFuncAttributeMaxDynamicSharedMemorySize };
+enum hipDeviceAttribute_t { hipDeviceAttributeMultiprocessorCount };
+inline hipError_t hipGetDevice(int* dev) { *dev = 0; return hipSuccess; }
+inline hipError_t hipDeviceGetAttribute(int* v, hipDeviceAttribute_t, int) { *v = 256; return hipSuccess; }
+inline hipError_t hipFuncSetAttribute(const void*, hipFuncAttribute, int) { return hipSuccess; }
+inline hipError_t hipGetLastError() { return hipSuccess; }
+inline hipError_t hipGetSymbolAddress(void** p, const void* symbol) { *p = const_cast<void*>(symbol); return hipSuccess; }
+#define HIP_SYMBOL(x) (&(x))
+#define __device__
+#define __align__(n) __attribute__((aligned(n)))
+#define hipLaunchKernelGGL(kern, grid, block, lds_bytes, stream, ...) \
+  ::hwsim::run_grid(grid, (int)(block).x, lds_bytes, [&]() { kern(__VA_ARGS__); })
+
 namespace hwsim {
 
 enum Op { OP_NONE, OP_DONE, OP_BARRIER, OP_MFMA32, OP_MFMA16, OP_TR, OP_SHFL, OP_WAVESYNC };

@@ -117,3 +117,36 @@ def test_reference_package_name_resolves_to_this_implementation():
     assert flag_attn.flash is flagattention_amd.flash and flag_attn.testing is flagattention_amd.testing
     assert callable(philox_cuda_seed_offset) and callable(recompute_mask)
     assert callable(flag_attn.flash.get_fwd_config) and callable(flag_attn.flash.get_bwd_config)
+
+
+def test_config_hook_resolution():
+    """The tile hooks (flash.py:290,493 of the reference) are called with the launch's shape; a compiled
+    tile is taken, anything else falls back to the default with one warning per distinct answer, and a
+    malformed answer is an assertion like the reference's shape checks."""
+    import warnings
+    from flagattention_amd import _config
+    compiled = ((128, 64), (256, 64))
+    seen_args = []
+
+    def hook(*a):
+        seen_args.append(a)
+        return (256, 64, 1, 4)
+    assert _config.resolve(hook, compiled, "t1", (1, 2, 3, 4, 128, True)) == (256, 64)
+    assert seen_args == [(1, 2, 3, 4, 128, True)]
+    with warnings.catch_warnings(record=True) as w:
+        warnings.simplefilter("always")
+        assert _config.resolve(lambda *a: (32, 32, 1, 4), compiled, "t2", (1,) * 6) == (128, 64)
+        assert _config.resolve(lambda *a: (32, 32, 1, 4), compiled, "t2", (1,) * 6) == (128, 64)
+        assert _config.resolve(lambda *a: (16, 32, 1, 4), compiled, "t2", (1,) * 6) == (128, 64)
+    assert len(w) == 2 and all(issubclass(x.category, RuntimeWarning) for x in w)
+    with pytest.raises(AssertionError):
+        _config.resolve(lambda *a: (128, 64), compiled, "t3", (1,) * 6)
+    with pytest.raises(AssertionError):
+        _config.resolve(lambda *a: (0, 64, 1, 4), compiled, "t3", (1,) * 6)
+
+
+def test_default_hooks_name_compiled_tiles():
+    from flagattention_amd import flash, piecewise
+    for mod in (flash, piecewise):
+        assert mod.get_fwd_config(1, 1, 4096, 4096, 128, True)[:2] in mod.FWD_TILES
+        assert mod.get_bwd_config(1, 1, 4096, 4096, 128, True)[:2] in mod.BWD_TILES

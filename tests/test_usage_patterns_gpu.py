@@ -57,14 +57,26 @@ def test_auxiliary_outputs_come_as_a_five_tuple():
         check(name, h, s, r)
 
 
-def test_replaced_config_hook_is_tolerated(monkeypatch):
-    """examples/use_cutom_config_func.py: callers may assign ``flash.get_fwd_config``.  Tile shapes are
-    compiled into the kernels here, so the hook changes nothing, but assigning it must not break."""
+def test_replaced_config_hook_is_called_and_reported(monkeypatch):
+    """examples/use_cutom_config_func.py: callers may assign ``flash.get_fwd_config``.  The hook is
+    called before the launch like in the reference (flash.py:64-66); a tile that no compiled kernel has
+    is reported once and the default tile is launched, with correct results."""
+    import warnings
     from flag_attn import flash
-    monkeypatch.setattr(flash, "get_fwd_config", lambda B, H, M, N, D, causal: (64, 64, 1, 4))
+    calls = []
+
+    def hook(B, H, M, N, D, causal):
+        calls.append((B, H, M, N, D, causal))
+        return (64, 64, 1, 4)
+    monkeypatch.setattr(flash, "get_fwd_config", hook)
     B, H, T, D = 2, 16, 1024, 128
     q, k, v = (torch.randn(B, H, T, D, dtype=torch.bfloat16, device="cuda:0", requires_grad=True) for _ in range(3))
-    o = flag_attn.flash_attention(q, k, v, causal=True)
+    with warnings.catch_warnings(record=True) as seen:
+        warnings.simplefilter("always")
+        o = flag_attn.flash_attention(q, k, v, causal=True)
+        flag_attn.flash_attention(q, k, v, causal=True)
+    assert calls == [(B, H, T, T, D, True)] * 2
+    assert len([w for w in seen if "BLOCK_M=64, BLOCK_N=64" in str(w.message)]) <= 1   # once per distinct answer
     go = torch.randn_like(o)
     grads = torch.autograd.grad(o, (q, k, v), go)
     g_ref = torch.autograd.grad(oracle_flash(q, k, v, True, upcast=True), (q, k, v), go)
