@@ -52,6 +52,9 @@ def check(code, what):
         raise AssertionError(f"{what}: argument rejected by the kernel library")
     if code == -2:
         raise AssertionError(f"{what}: configuration not supported by the kernel library")
+    if code == -3:
+        raise AssertionError(f"{what}: the launch needs more scratch memory than the library's static device "
+                             "array holds (FA_STATIC_SCRATCH_BYTES); use the entry point that takes a workspace")
     raise KernelError(f"{what}: HIP error {code}")
 
 
@@ -228,6 +231,22 @@ def paged_attn_balanced(lib, out, query, key_cache, value_cache, context_lens, b
                                   float(scale), num_seqs, Hq, Hkv, D, block_size, ptr(workspace),
                                   workspace.numel() * workspace.element_size(), int(num_workgroups),
                                   stream_of(query)), "paged_attn_balanced")
+
+
+def paged_attn_balanced_static(lib, out, query, key_cache, value_cache, context_lens, block_tables, scale,
+                               num_workgroups):
+    """paged_attn_balanced on the library's static device scratch: allocates nothing."""
+    num_seqs, Hq, D = query.shape
+    _, Hkv, block_size, _ = key_cache.shape
+    assert block_tables.dtype in (torch.int32, torch.int64)
+    check(lib.paged_attn_balanced_static(dtype_code(query), ptr(out), out.stride(0), out.stride(1),
+                                         ptr(query), query.stride(0), query.stride(1),
+                                         ptr(key_cache), ptr(value_cache),
+                                         key_cache.stride(0), key_cache.stride(1), key_cache.stride(2),
+                                         ptr(context_lens), ptr(block_tables),
+                                         int(block_tables.dtype == torch.int64), block_tables.stride(0),
+                                         float(scale), num_seqs, Hq, Hkv, D, block_size, int(num_workgroups),
+                                         stream_of(query)), "paged_attn_balanced_static")
 
 
 def paged_reduce(lib, out, tmp_out, max_logits, exp_sums, context_lens, Hkv, partition_size, num_parts):

@@ -46,7 +46,11 @@ SIGNATURES = {
     "paged_attn_balanced_workspace": [_i, _i],
     "paged_attn_balanced": [_i, _p, _i64, _i64, _p, _i64, _i64, _p, _p, _i64, _i64, _i64, _p, _p, _i, _i64,
                             _f, _i, _i, _i, _i, _i, _p, _i64, _i, _p],
+    "paged_attn_balanced_static": [_i, _p, _i64, _i64, _p, _i64, _i64, _p, _p, _i64, _i64, _i64, _p, _p, _i, _i64,
+                                   _f, _i, _i, _i, _i, _i, _i, _p],
 }
+
+STATIC_SCRATCH_BYTES = 17 * 1024 * 1024   # FA_STATIC_SCRATCH_BYTES of include/flagattn.h
 
 
 def bind(path, names=None):

@@ -4,6 +4,8 @@
 #include "../../include/flagattn.h"
 #include "params.hpp"
 
+#include <atomic>
+
 namespace {
 
 constexpr int kVersion = 1;
@@ -32,14 +34,10 @@ extern "C" {
 int fa_version(void) { return kVersion; }
 
 int fa_num_cus(void) {
-#ifdef FLAGATTN_HOST_SIM
-  return 256;
-#else
   int dev = 0, n = 0;
   if (hipGetDevice(&dev) != hipSuccess) return -1;
   if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return -1;
   return n;
-#endif
 }
 
 int fa_fwd(int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v, const fa_view4* o,
@@ -359,6 +357,56 @@ int paged_attn_balanced(int dtype, void* out, int64_t o_stride_s, int64_t o_stri
   p.scale = attn_scale; p.block_size = block_size;
   p.ws = (float*)workspace; p.num_wgs = num_workgroups;
   return fa::run_paged_balanced(p, (hipStream_t)stream);
+}
+
+// ---------------------------------------------------------------------------------------------
+// paged_attn_balanced without a caller-provided workspace: the partial-result slots and the
+// per-workgroup records live in a device array that is part of the library's code object.
+// ---------------------------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[FA_STATIC_SCRATCH_BYTES];
+
+namespace {
+// The array's name is only a host-side handle; each device that loads the library holds its own copy
+// at its own address, looked up once per device (with that device current) and kept here.
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_of_device[kMaxDevices];
+
+int scratch_of_current_device(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= kMaxDevices) return FA_ERR_UNSUPPORTED;
+  void* ptr = g_scratch_of_device[dev].load(std::memory_order_acquire);
+  if (!ptr) {  // first call on this device; a concurrent first call looks up the same address
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (!ptr) return FA_ERR_UNSUPPORTED;
+    g_scratch_of_device[dev].store(ptr, std::memory_order_release);
+  }
+  *out = ptr;
+  return 0;
+}
+}  // namespace
+
+int paged_attn_balanced_static(int dtype, void* out, int64_t o_stride_s, int64_t o_stride_h, const void* query,
+                               int64_t q_stride_s, int64_t q_stride_h, const void* key_cache,
+                               const void* value_cache, int64_t kv_stride_blk, int64_t kv_stride_h,
+                               int64_t kv_stride_tok, const int32_t* context_lens, const void* block_tables,
+                               int bt_is_int64, int64_t bt_stride, float attn_scale, int num_seqs,
+                               int num_q_heads, int num_kv_heads, int head_size, int block_size,
+                               int num_workgroups, void* stream) {
+  if (num_workgroups <= 0 || head_size <= 0) return FA_ERR_BAD_ARGUMENT;
+  const int64_t need = fa::paged_balanced_workspace_bytes(num_workgroups, head_size);
+  if (need > (int64_t)FA_STATIC_SCRATCH_BYTES) return FA_ERR_SCRATCH_TOO_SMALL;
+  void* ws = nullptr;
+  const int rc = scratch_of_current_device(&ws);
+  if (rc) return rc;
+  // nothing in the scratch has to start at zero: every slot and record that the merge kernel reads was
+  // written by the attention kernel of the same call
+  return paged_attn_balanced(dtype, out, o_stride_s, o_stride_h, query, q_stride_s, q_stride_h, key_cache,
+                             value_cache, kv_stride_blk, kv_stride_h, kv_stride_tok, context_lens,
+                             block_tables, bt_is_int64, bt_stride, attn_scale, num_seqs, num_q_heads,
+                             num_kv_heads, head_size, block_size, ws, need, num_workgroups, stream);
 }
 
 int paged_reduce(int dtype, void* out, int64_t o_stride_s, int64_t o_stride_h, const void* tmp_out,

@@ -29,6 +29,7 @@ extern "C" {
 
 #define FA_ERR_BAD_ARGUMENT (-1)
 #define FA_ERR_UNSUPPORTED (-2)
+#define FA_ERR_SCRATCH_TOO_SMALL (-3) /* paged_attn_balanced_static: the launch needs more than FA_STATIC_SCRATCH_BYTES */
 
 typedef struct fa_view4 {
   void* ptr;
@@ -202,6 +203,28 @@ int paged_attn_balanced(int dtype, void* out, int64_t o_stride_s, int64_t o_stri
                         int bt_is_int64, int64_t bt_stride, float attn_scale, int num_seqs,
                         int num_q_heads, int num_kv_heads, int head_size, int block_size,
                         void* workspace, int64_t workspace_bytes, int num_workgroups, void* stream);
+
+/* paged_attn_balanced_static: paged_attn_balanced for callers that cannot allocate device memory --
+ * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
+ * counterpart in the reference (whose wrapper allocates its partition buffers with torch,
+ * paged.py:92-108).  Same arguments and same result as paged_attn_balanced minus the workspace: the
+ * partial-result slots live in a device array of FA_STATIC_SCRATCH_BYTES inside the library, which
+ * every device that runs the library holds until the process ends.  The call allocates and frees
+ * nothing (the array's device address is looked up on the first call on each device).  A launch whose
+ * paged_attn_balanced_workspace(num_workgroups, head_size) exceeds FA_STATIC_SCRATCH_BYTES is rejected
+ * with FA_ERR_SCRATCH_TOO_SMALL and nothing is launched (the array holds 1024 workgroups at head_size
+ * <= 128 and 256 workgroups at head_size 512: more than one resident wave of a 256-CU device).  All calls on
+ * one device share the one array: calls that may overlap on a device (different streams, or threads
+ * that do not order their launches) race on it and must use paged_attn_balanced with separate
+ * workspaces instead. */
+#define FA_STATIC_SCRATCH_BYTES (17 * 1024 * 1024)
+int paged_attn_balanced_static(int dtype, void* out, int64_t o_stride_s, int64_t o_stride_h, const void* query,
+                               int64_t q_stride_s, int64_t q_stride_h, const void* key_cache,
+                               const void* value_cache, int64_t kv_stride_blk, int64_t kv_stride_h,
+                               int64_t kv_stride_tok, const int32_t* context_lens, const void* block_tables,
+                               int bt_is_int64, int64_t bt_stride, float attn_scale, int num_seqs,
+                               int num_q_heads, int num_kv_heads, int head_size, int block_size,
+                               int num_workgroups, void* stream);
 
 #ifdef __cplusplus
 }

@@ -387,6 +387,40 @@ def test_paged_attention_balanced(lib, seqs, Hq, G, D, bs, lens, wgs, dtype, tdt
         assert torch.allclose(out[live], ref, atol=2e-3, rtol=1e-5)
 
 
+def test_paged_attention_balanced_static_scratch(lib):
+    """The entry point without a workspace argument (static scratch inside the library) against the one
+    with a caller-provided workspace: bit-equal, on two calls in a row, the second one smaller, with the
+    scratch still holding the first call's partial results; and the size limit is enforced."""
+    from flagattention_amd import _lib
+    calls = [  # seqs, Hq, G, D, block, lens, workgroups
+        (4, 4, 2, 64, 16, [700, 1, 300, 129], 7),
+        (2, 4, 2, 64, 16, [130, 260], 3),
+    ]
+    for seqs, Hq, G, D, bs, lens, wgs in calls:
+        Hk = Hq // G
+        lens = torch.tensor(lens, dtype=torch.int32)
+        nb, sc = 60, D ** -0.5
+        q = torch.empty(seqs, Hq, D).uniform_(-sc, sc).to(torch.float16)
+        kc = torch.empty(nb, Hk, bs, D).uniform_(-sc, sc).to(torch.float16)
+        vc = torch.empty(nb, Hk, bs, D).uniform_(-sc, sc).to(torch.float16)
+        bt = torch.randint(0, nb, (seqs, (int(lens.max()) + bs - 1) // bs))
+        out_ws = torch.full_like(q, float("nan"))
+        ws = torch.full((lib.paged_attn_balanced_workspace(wgs, D) // 4,), float("nan"))
+        _abi.paged_attn_balanced(lib, out_ws, q, kc, vc, lens, bt, sc, ws, wgs)
+        out_static = torch.full_like(q, float("nan"))
+        _abi.paged_attn_balanced_static(lib, out_static, q, kc, vc, lens, bt, sc, wgs)
+        assert torch.equal(out_ws, out_static)
+        ref = paged_attention(q, kc, vc, bt, lens, sc)
+        assert torch.allclose(out_static, ref, atol=2e-3, rtol=1e-5)
+    # 4096 workgroups at head size 64 need 4096 * 8464 bytes: more than the array holds
+    assert lib.paged_attn_balanced_workspace(4096, D) > _lib.STATIC_SCRATCH_BYTES
+    with pytest.raises(AssertionError, match="scratch"):
+        _abi.paged_attn_balanced_static(lib, out_static, q, kc, vc, lens, bt, sc, 4096)
+    # the sizes the host wrapper launches fit: one resident wave of a 256-CU device
+    assert lib.paged_attn_balanced_workspace(512, 128) <= _lib.STATIC_SCRATCH_BYTES
+    assert lib.paged_attn_balanced_workspace(256, 512) <= _lib.STATIC_SCRATCH_BYTES
+
+
 def test_entry_points_reject_bad_arguments(lib):
     q = rnd((1, 2, 32, 64), torch.float16)
     k = rnd((1, 2, 32, 64), torch.float16)
