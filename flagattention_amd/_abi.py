@@ -77,12 +77,13 @@ def _u64(x):
     return int(x) & 0xFFFFFFFFFFFFFFFF
 
 
-def fa_fwd(lib, q, k, v, o, lse, causal, sm_scale, dropout=NO_DROPOUT):
+def fa_fwd(lib, q, k, v, o, lse, causal, sm_scale, dropout=NO_DROPOUT, block_m=0):
+    """block_m: query rows per workgroup (128 or 256), 0 = the library's choice."""
     B, H, M, D = q.shape
     Hk, N = k.shape[1], k.shape[2]
     check(lib.fa_fwd(dtype_code(q), view4(q), view4(k), view4(v), view4(o), ptr(lse),
                      B, H, Hk, M, N, D, int(causal), float(sm_scale), float(dropout[0]), _u64(dropout[1]),
-                     _u64(dropout[2]), stream_of(q)), "fa_fwd")
+                     _u64(dropout[2]), int(block_m), stream_of(q)), "fa_fwd")
 
 
 def pw_fwd(lib, q1, k1, q2, k2, v, o, lse, w, causal, sm_scale):

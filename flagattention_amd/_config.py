@@ -12,6 +12,12 @@ import warnings
 _warned = set()
 
 
+def warn_once(key, message):
+    if key not in _warned:
+        _warned.add(key)
+        warnings.warn(message, RuntimeWarning, stacklevel=3)
+
+
 def resolve(hook, compiled, what, args):
     """Calls ``hook(*args)`` -> (BLOCK_M, BLOCK_N, num_stages, num_warps) and returns the
     (BLOCK_M, BLOCK_N) to launch: the hook's if it is in ``compiled`` (a sequence whose first entry is

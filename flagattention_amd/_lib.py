@@ -23,7 +23,7 @@ _v = ctypes.POINTER(View4)
 SIGNATURES = {
     "fa_version": [],
     "fa_num_cus": [],
-    "fa_fwd": [_i, _v, _v, _v, _v, _p, _i, _i, _i, _i, _i, _i, _i, _f, _f, _u64, _u64, _p],
+    "fa_fwd": [_i, _v, _v, _v, _v, _p, _i, _i, _i, _i, _i, _i, _i, _f, _f, _u64, _u64, _i, _p],
     "fa_bwd_delta": [_i, _v, _v, _p, _i, _i, _i, _i, _p],
     "fa_bwd_dkdv": [_i, _v, _v, _v, _v, _p, _p, _v, _v, _i, _i, _i, _i, _i, _i, _i, _i, _f, _f, _u64, _u64, _p],
     "fa_bwd_dq": [_i, _v, _v, _v, _v, _p, _p, _v, _i, _i, _i, _i, _i, _i, _i, _f, _f, _u64, _u64, _p],

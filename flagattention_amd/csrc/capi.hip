@@ -42,7 +42,7 @@ int fa_num_cus(void) {
 
 int fa_fwd(int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v, const fa_view4* o,
            float* lse, int B, int H, int Hk, int M, int N, int D, int causal, float sm_scale,
-           float dropout_p, uint64_t seed, uint64_t offset, void* stream) {
+           float dropout_p, uint64_t seed, uint64_t offset, int block_m, void* stream) {
   if (!view_ok(q) || !view_ok(k) || !view_ok(v) || !view_ok(o) || !lse) return FA_ERR_BAD_ARGUMENT;
   if (!head_dim_ok(D)) return FA_ERR_UNSUPPORTED;
   if (Hk <= 0 || H % Hk) return FA_ERR_BAD_ARGUMENT;
@@ -53,6 +53,7 @@ int fa_fwd(int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v, c
   p.group = H / Hk;
   p.causal = causal; p.w = 0; p.sm_scale = sm_scale; p.dtype = dtype;
   p.dropout_p = dropout_p; p.seed = seed; p.offset = offset;
+  p.block_m = block_m;
   return fa::run_fwd(p, false, (hipStream_t)stream);
 }
 

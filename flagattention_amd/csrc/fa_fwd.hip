@@ -271,9 +271,24 @@ static int dispatch_fwd(const FwdParams& p, bool piecewise, hipStream_t stream) 
   return p.dropout_p > 0.f ? launch_fwd<T, false, true>(p, stream) : launch_fwd<T, false, false>(p, stream);
 }
 
+// Which kernel a launch without an explicit tile takes: the 256-row kernel is the faster one per tile,
+// but its workgroups hold a compute unit alone, so it needs at least one workgroup per compute unit.
+static bool prefer_wide(const FwdParams& p) {
+  static int num_cus = 0;   // one device kind per process
+  if (num_cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return false;
+    num_cus = n;
+  }
+  return (int64_t)((p.M + 255) / 256) * p.H * p.B >= num_cus;
+}
+
 int run_fwd(const FwdParams& p, bool piecewise, hipStream_t stream) {
   if (p.B <= 0 || p.H <= 0 || p.M <= 0 || p.N < 0 || p.group <= 0) return kBadArgument;
   if (!(p.dropout_p >= 0.f && p.dropout_p < 1.f) || (piecewise && p.dropout_p > 0.f)) return kBadArgument;
+  if (p.block_m != 0 && p.block_m != 128 && p.block_m != 256) return kUnsupported;
+  if (p.block_m == 256 && (piecewise || !fwd_wide_supported(p))) return kUnsupported;
+  if (!piecewise && (p.block_m == 256 || (p.block_m == 0 && fwd_wide_supported(p) && prefer_wide(p)))) return run_fwd_wide(p, stream);
   if (p.dtype == kDtypeF16) return dispatch_fwd<hw::half_t>(p, piecewise, stream);
   if (p.dtype == kDtypeBF16) return dispatch_fwd<hw::bf16_t>(p, piecewise, stream);
   return kUnsupported;

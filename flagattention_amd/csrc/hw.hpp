@@ -43,6 +43,9 @@ FA_DEVICE int block_z() { return (int)blockIdx.z; }
 FA_DEVICE int grid_x() { return (int)gridDim.x; }
 FA_DEVICE int grid_z() { return (int)gridDim.z; }
 FA_DEVICE void block_sync() { __syncthreads(); }
+// The workgroup barrier alone, without the memory fence of block_sync(): for code that has already
+// waited for the accesses it needs ordered.
+FA_DEVICE void barrier_only() { __builtin_amdgcn_s_barrier(); }
 // Orders the LDS traffic of one wavefront: writes issued by any lane before the call are visible
 // to reads issued by any lane after it (LDS serves a wavefront's requests in order; this only stops
 // the compiler from moving accesses across).
@@ -74,6 +77,118 @@ FA_DEVICE f32x16 mfma32_vacc(bf16x8 a, bf16x8 b, f32x16 c) {
   asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
   return c;
 }
+// First product of a chain with the accumulator pinned to VGPRs: D = A * B (no accumulator to read).
+FA_DEVICE f32x16 mfma32_vacc_first(half8 a, half8 b) {
+  f32x16 c;
+  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "a"(b));
+  return c;
+}
+FA_DEVICE f32x16 mfma32_vacc_first(bf16x8 a, bf16x8 b) {
+  f32x16 c;
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "a"(b));
+  return c;
+}
+// The product with the accumulator pinned to AGPRs and both operands in VGPRs (an output accumulator
+// that the vector ALU touches only in rare rescales and at the end).  As with mfma32_vacc the compiler
+// does not know that this is a matrix instruction: a CALLER that reads the accumulator with ordinary
+// code afterwards first lets the pipe drain (mfma_drain()).
+FA_DEVICE void mfma32_aacc(half8 a, half8 b, f32x16& c) {
+  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+FA_DEVICE void mfma32_aacc(bf16x8 a, bf16x8 b, f32x16& c) {
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
+// Chain instructions with accumulator and both operands in VGPRs.
+FA_DEVICE f32x16 mfma32_vvv_first(half8 a, half8 b) {
+  f32x16 c;
+  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
+  return c;
+}
+FA_DEVICE f32x16 mfma32_vvv_first(bf16x8 a, bf16x8 b) {
+  f32x16 c;
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
+  return c;
+}
+FA_DEVICE f32x16 mfma32_vvv(half8 a, half8 b, f32x16 c) {
+  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+  return c;
+}
+FA_DEVICE f32x16 mfma32_vvv(bf16x8 a, bf16x8 b, f32x16 c) {
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+  return c;
+}
+// Chain instructions with both operands in AGPRs (LDS reads can target AGPRs directly; a register-resident
+// operand is moved there once) and the accumulator in VGPRs.
+// (the first product of a chain names its accumulator as read-write although it only writes it: the
+// accumulator then stays one long-lived value in one place for the register allocator)
+FA_DEVICE void mfma32_vaa_first(half8 a, half8 b, f32x16& c) {
+  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "+v"(c) : "a"(a), "a"(b));
+}
+FA_DEVICE void mfma32_vaa_first(bf16x8 a, bf16x8 b, f32x16& c) {
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "+v"(c) : "a"(a), "a"(b));
+}
+FA_DEVICE void mfma32_vaa(half8 a, half8 b, f32x16& c) {
+  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "a"(a), "a"(b));
+}
+FA_DEVICE void mfma32_vaa(bf16x8 a, bf16x8 b, f32x16& c) {
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "a"(a), "a"(b));
+}
+// Accumulator and A operand in AGPRs, B operand in VGPRs.
+FA_DEVICE void mfma32_aav(half8 a, half8 b, f32x16& c) {
+  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "a"(a), "v"(b));
+}
+FA_DEVICE void mfma32_aav(bf16x8 a, bf16x8 b, f32x16& c) {
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "a"(a), "v"(b));
+}
+// The same two chain instructions with the accumulator in AGPRs (B operand in AGPRs as well).
+FA_DEVICE f32x16 mfma32_aacc_first(half8 a, half8 b) {
+  f32x16 c;
+  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&a"(c) : "v"(a), "a"(b));
+  return c;
+}
+FA_DEVICE f32x16 mfma32_aacc_first(bf16x8 a, bf16x8 b) {
+  f32x16 c;
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&a"(c) : "v"(a), "a"(b));
+  return c;
+}
+FA_DEVICE f32x16 mfma32_aacc_ab(half8 a, half8 b, f32x16 c) {
+  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "a"(b));
+  return c;
+}
+FA_DEVICE f32x16 mfma32_aacc_ab(bf16x8 a, bf16x8 b, f32x16 c) {
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "a"(b));
+  return c;
+}
+// max(a, b, c) and max(a, b) as single instructions (no canonicalisation of the inputs: callers pass
+// matrix-instruction results and values derived from them)
+FA_DEVICE float max3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+FA_DEVICE float max2(float a, float b) {
+  float r;
+  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+// Element access to an accumulator that lives in AGPRs, spelled out so that the compiler never sees a
+// vector-ALU use of it (which would make it keep the accumulator in VGPRs and copy it around every
+// matrix instruction).
+template <int R> FA_DEVICE float acc_read(const f32x16& c) {
+  float x;
+  asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(x) : "a"(c[R]));
+  return x;
+}
+template <int R> FA_DEVICE void acc_scale(f32x16& c, float f) {
+  float t;
+  asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 1\n\tv_accvgpr_write_b32 %0, %1"
+               : "+a"(c[R]), "=&v"(t) : "v"(f));
+}
+template <int R> FA_DEVICE void acc_clear(f32x16& c) {
+  asm volatile("v_accvgpr_write_b32 %0, 0" : "=a"(c[R]));
+}
+// More wait states than any matrix instruction needs before its result may be read by other units.
+FA_DEVICE void mfma_drain() { asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 7" ::: "memory"); }
 // Moves a register-resident operand to AGPRs for good (what mfma32_vacc takes as B).
 template <class V>
 FA_DEVICE void keep_in_agprs(V& v) { asm volatile("" : "+a"(v)); }
@@ -96,6 +211,15 @@ FA_DEVICE short4v lds_read_tr16(const void* lds_ptr) {
       (__attribute__((address_space(3))) short4v*)(uintptr_t)lds_ptr);
 }
 
+// LDS accesses by byte address (as returned by lds_address()): the address arithmetic stays in
+// 32-bit registers and constant parts fold into the instruction's offset field.
+FA_DEVICE u32x4 lds_load16(uint32_t addr) {
+  return *(const __attribute__((address_space(3))) u32x4*)(uintptr_t)addr;
+}
+FA_DEVICE short4v lds_read_tr16_at(uint32_t addr) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) short4v*)(uintptr_t)addr);
+}
+
 // True in every lane if the predicate holds in any lane of the wavefront.
 FA_DEVICE bool wave_any(bool pred) { return __builtin_amdgcn_ballot_w64(pred) != 0; }
 
@@ -103,6 +227,15 @@ FA_DEVICE bool wave_any(bool pred) { return __builtin_amdgcn_ballot_w64(pred) !=
 FA_DEVICE float xor32(float x) { return __shfl_xor(x, 32, 64); }
 // Value held by lane (l ^ mask) for mask < 64.
 FA_DEVICE float shfl_xor(float x, int mask) { return __shfl_xor(x, mask, 64); }
+
+// Exchanges the upper 32 lanes of a with the lower 32 lanes of b (one instruction):
+//   a' = [a.lo, b.lo],  b' = [a.hi, b.hi]
+FA_DEVICE void swap_halves(float& a, float& b) {
+  // written as assembly: the compiler's lowering of the corresponding builtin returns the first result
+  // for both halves of its result pair.  The wait states around it are the ones the compiler places
+  // around the instruction itself (vector-ALU results feeding it, its results feeding the vector ALU).
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
 
 // Tells the compiler that x has the same value in every lane (kept in a scalar register).
 FA_DEVICE int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
@@ -112,6 +245,20 @@ FA_DEVICE int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
 FA_DEVICE void store_streaming(void* p, u32x4 v) { __builtin_nontemporal_store(v, (u32x4*)p); }
 FA_DEVICE u32x4 load_streaming(const void* p) { return __builtin_nontemporal_load((const u32x4*)p); }
 
+// 16 bytes per lane from global memory straight into LDS, no register in between: lane i's bytes land
+// at LDS byte address lds_base + 16 i (lds_base wave-uniform, a multiple of 16); the source address is
+// base (wave-uniform) + lane_offset bytes.  Completion is counted like any global load
+// (wait_global_loads()); the compiler is not told that LDS changes, so the caller orders the LDS reads
+// of that region behind the wait and a barrier itself.
+FA_DEVICE void dma_load16(const void* base, uint32_t lane_offset, uint32_t lds_base) {
+  // (one wait state between the scalar write of M0 and the instruction that reads it)
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(lane_offset), "s"(base), "s"(lds_base) : "memory", "m0");
+}
+// LDS byte address of a pointer into the workgroup's LDS allocation.
+FA_DEVICE uint32_t lds_address(const void* p) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
+}
+
 // Waits until every global load issued so far has delivered its registers.  Placed between the
 // loads of loop-invariant operands and a loop that also prefetches: otherwise the compiler puts the
 // wait at the operands' first use INSIDE the loop, where it also covers the prefetch just issued.
@@ -120,6 +267,12 @@ FA_DEVICE void wait_global_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // v
 // Marks a branch body as not speculatable, so that a wavefront-uniform `if` stays a branch instead
 // of being turned into unconditional arithmetic on selected operands.
 FA_DEVICE void keep_branch() { asm volatile("" ::: "memory"); }
+
+// Makes the compiler materialise x at this point of the instruction stream: the scheduling fence only
+// binds the instruction scheduler, while earlier passes sink a side-effect-free computation towards its
+// first use, across fences and branches.  Costs no instruction.
+FA_DEVICE void pin(float& x) { asm volatile("" : "+v"(x)); }
+FA_DEVICE void pin(uint32_t& x) { asm volatile("" : "+v"(x)); }
 
 // Nothing is scheduled across this point by the compiler (software-pipelining fence).
 FA_DEVICE void sched_fence() { __builtin_amdgcn_sched_barrier(0); }
@@ -141,7 +294,30 @@ FA_DEVICE void sched_prefetched_operands() {
 FA_DEVICE float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
 FA_DEVICE float log_nat(float x) { return __logf(x); }
 
+// Two fp32 values rounded to T and packed (lo = a, hi = b), and acc + lo + hi of such a pair.
+FA_DEVICE uint32_t pack2(half_t, float a, float b) {
+  typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+  h2 v; v[0] = (_Float16)a; v[1] = (_Float16)b;
+  return __builtin_bit_cast(uint32_t, v);
+}
+FA_DEVICE uint32_t pack2(bf16_t, float a, float b) {
+  typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+  b2 v; v[0] = (__bf16)a; v[1] = (__bf16)b;
+  return __builtin_bit_cast(uint32_t, v);
+}
+FA_DEVICE float add_pair(half_t, uint32_t pair, float acc) {
+  typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+  h2 one; one[0] = (_Float16)1.f; one[1] = (_Float16)1.f;
+  return __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, pair), one, acc, false);
+}
+FA_DEVICE float add_pair(bf16_t, uint32_t pair, float acc) {
+  typedef __bf16 b2 __attribute__((ext_vector_type(2)));
+  b2 one; one[0] = (__bf16)1.f; one[1] = (__bf16)1.f;
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(b2, pair), one, acc, false);
+}
+
 }  // namespace hw
+#include "pinned_regs.hpp"
 #endif  // FLAGATTN_HOST_SIM
 
 namespace hw {

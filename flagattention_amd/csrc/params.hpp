@@ -23,6 +23,7 @@ struct FwdParams {
   int dtype;
   float dropout_p;        // 0 = no dropout; otherwise the mask is drawn from (seed, offset)
   uint64_t seed, offset;
+  int block_m;            // query rows per workgroup: 128, 256, or 0 = the library's choice
 };
 
 struct BwdParams {
@@ -61,6 +62,8 @@ struct TotalParams {
 
 namespace fa {
 int run_fwd(const FwdParams& p, bool piecewise, hipStream_t stream);
+bool fwd_wide_supported(const FwdParams& p);   // the 256-row kernel (fa_fwd_wide.hip) can serve this launch
+int run_fwd_wide(const FwdParams& p, hipStream_t stream);
 int run_bwd_delta(const BwdParams& p, hipStream_t stream);
 int run_bwd_dkdv(const BwdParams& p, bool piecewise, hipStream_t stream);
 int run_bwd_dq(const BwdParams& p, bool piecewise, hipStream_t stream);

@@ -21,9 +21,15 @@ __all__ = ["attention"]
 _HEAD_DIMS = (16, 32, 64, 128)
 
 
-# (BLOCK_M, BLOCK_N) the kernels are compiled for; the first entry is the default
-FWD_TILES = ((128, 64),)
+# (BLOCK_M, BLOCK_N) the kernels are compiled for; the first entry is the fallback
+FWD_TILES = ((128, 64), (256, 64))
 BWD_TILES = ((64, 128),)
+
+
+def wide_forward_applies(D, dropout_p=0.0):
+    """The 256-row forward kernel (64 query rows per wavefront, one wavefront per SIMD) is built for
+    head size 128 without dropout."""
+    return D == 128 and not dropout_p > 0
 
 
 def get_fwd_config(B, H, M, N, D, causal):
@@ -32,8 +38,22 @@ def get_fwd_config(B, H, M, N, D, causal):
 
     An overridable module-level hook like ``src/flag_attn/flash.py:290-322``, called before every
     forward launch (``flash.py:64-66``).  The kernels are compiled ahead of time, so an override may
-    only choose among ``FWD_TILES``; any other answer is reported once and the default is launched."""
+    only choose among ``FWD_TILES``; any other answer is reported once and the fallback is launched.
+    The default takes the 256-row kernel where it applies and the launch has at least one workgroup
+    per compute unit (its workgroups hold a compute unit alone)."""
+    if wide_forward_applies(D) and -(-M // 256) * H * B >= _num_cus():
+        return (256, 64, 5, 4)
     return (128, 64, 2, 4)
+
+
+_NUM_CUS = {}
+
+
+def _num_cus():
+    dev = torch.cuda.current_device() if torch.cuda.is_available() else -1
+    if dev not in _NUM_CUS:
+        _NUM_CUS[dev] = _lib.get().fa_num_cus() if dev >= 0 else 256
+    return _NUM_CUS[dev]
 
 
 def get_bwd_config(B, H, M, N, D, causal):
@@ -76,12 +96,18 @@ class FlashAttention(torch.autograd.Function):
                 o, L = split_kv_forward(lib, q, k, v, causal, sm_scale, splits)
             else:
                 # looked up by name at call time, so that an assignment to flash.get_fwd_config takes effect
-                _config.resolve(get_fwd_config, FWD_TILES, "flash_attention forward", (B, H, M, N, D, causal))
+                block_m, _ = _config.resolve(get_fwd_config, FWD_TILES, "flash_attention forward",
+                                             (B, H, M, N, D, causal))
+                if block_m == 256 and not (wide_forward_applies(D, dropout_p) and sm_scale > 0):
+                    _config.warn_once(("fwd-wide", D, is_dropout),
+                                      "flash_attention forward: the 256-row kernel is built for head size 128 "
+                                      "without dropout; launching the 128-row kernel")
+                    block_m = 128
                 o = torch.empty_like(q)
                 if not _abi.is_kernel_ready(o):
                     o = torch.empty(q.shape, dtype=q.dtype, device=q.device)
                 L = torch.empty((B, H, M), device=q.device, dtype=torch.float32)
-                _abi.fa_fwd(lib, q, k, v, o, L, causal, sm_scale, dropout)
+                _abi.fa_fwd(lib, q, k, v, o, L, causal, sm_scale, dropout, block_m)
             tot_attn = None
             if return_total_attention:
                 tot_attn = _total_attention(lib, q, k, L, causal, sm_scale)

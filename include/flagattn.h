@@ -53,10 +53,16 @@ int fa_num_cus(void);
  * (flash.py:328-330); with dropout_p > 0 the probability of (b, h, m, n) enters the second product
  * only if the uniform number Triton's tl.rand(seed, offset + ((b H + h) M + m) N + n, n_rounds=6) would
  * give exceeds dropout_p, and o is scaled by 1 / (1 - dropout_p); lse is unaffected.  The backward
- * entry points below take the same three values and must be given the forward's. */
+ * entry points below take the same three values and must be given the forward's.
+ * block_m: the BLOCK_M of the reference's launch (flash.py:64-66, 84: query rows per workgroup, chosen
+ * by the overridable get_fwd_config).  Two kernels are compiled: 128 (every head size, dropout) and 256
+ * (head size 128 without dropout: 64 rows per wavefront, one wavefront per SIMD); 0 lets the library
+ * choose (256 where it applies and the launch has at least one workgroup per compute unit).  Any other
+ * value, or 256 where it does not apply, returns FA_ERR_UNSUPPORTED.  The results of the two kernels
+ * differ only in rounding. */
 int fa_fwd(int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v, const fa_view4* o,
            float* lse, int B, int H, int Hk, int M, int N, int D, int causal, float sm_scale,
-           float dropout_p, uint64_t seed, uint64_t offset, void* stream);
+           float dropout_p, uint64_t seed, uint64_t offset, int block_m, void* stream);
 
 /* ----------------------------------------------------------------- flash attention, backward --
  * The reference's three launches in FlashAttention.backward, src/flag_attn/flash.py:191-249:

@@ -219,6 +219,7 @@ inline void wait_global_loads() {}
 inline int uniform(int x) { return x; }
 inline int grid_z() { return hwsim::gz; }
 inline void block_sync() { hwsim::yield(hwsim::OP_BARRIER); }
+inline void barrier_only() { hwsim::yield(hwsim::OP_BARRIER); }
 inline void wave_sync() { hwsim::yield(hwsim::OP_WAVESYNC); }
 
 template <class V8> inline f32x16 mfma32_any(V8 a, V8 b, f32x16 c) {
@@ -233,6 +234,36 @@ template <class V8> inline f32x16 mfma32_any(V8 a, V8 b, f32x16 c) {
 }
 inline f32x16 mfma32(half8 a, half8 b, f32x16 c) { return mfma32_any(a, b, c); }
 inline f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) { return mfma32_any(a, b, c); }
+inline f32x16 zero16() { f32x16 z; for (int r = 0; r < 16; ++r) z[r] = 0.f; return z; }
+inline f32x16 mfma32_vacc_first(half8 a, half8 b) { return mfma32_any(a, b, zero16()); }
+inline f32x16 mfma32_vacc_first(bf16x8 a, bf16x8 b) { return mfma32_any(a, b, zero16()); }
+inline void mfma32_aacc(half8 a, half8 b, f32x16& c) { c = mfma32_any(a, b, c); }
+inline void mfma32_aacc(bf16x8 a, bf16x8 b, f32x16& c) { c = mfma32_any(a, b, c); }
+inline f32x16 mfma32_aacc_first(half8 a, half8 b) { return mfma32_any(a, b, zero16()); }
+inline f32x16 mfma32_aacc_first(bf16x8 a, bf16x8 b) { return mfma32_any(a, b, zero16()); }
+inline f32x16 mfma32_aacc_ab(half8 a, half8 b, f32x16 c) { return mfma32_any(a, b, c); }
+inline f32x16 mfma32_aacc_ab(bf16x8 a, bf16x8 b, f32x16 c) { return mfma32_any(a, b, c); }
+inline f32x16 mfma32_vvv_first(half8 a, half8 b) { return mfma32_any(a, b, zero16()); }
+inline f32x16 mfma32_vvv_first(bf16x8 a, bf16x8 b) { return mfma32_any(a, b, zero16()); }
+inline f32x16 mfma32_vvv(half8 a, half8 b, f32x16 c) { return mfma32_any(a, b, c); }
+inline f32x16 mfma32_vvv(bf16x8 a, bf16x8 b, f32x16 c) { return mfma32_any(a, b, c); }
+inline void mfma32_vaa_first(half8 a, half8 b, f32x16& c) { c = mfma32_any(a, b, zero16()); }
+inline void mfma32_vaa_first(bf16x8 a, bf16x8 b, f32x16& c) { c = mfma32_any(a, b, zero16()); }
+inline void mfma32_vaa(half8 a, half8 b, f32x16& c) { c = mfma32_any(a, b, c); }
+inline void mfma32_vaa(bf16x8 a, bf16x8 b, f32x16& c) { c = mfma32_any(a, b, c); }
+inline void mfma32_aav(half8 a, half8 b, f32x16& c) { c = mfma32_any(a, b, c); }
+inline void mfma32_aav(bf16x8 a, bf16x8 b, f32x16& c) { c = mfma32_any(a, b, c); }
+// accumulator tuples that the GPU build pins to fixed physical registers: plain values here
+template <int I, class V8> inline void pinned_o_mfma(V8 a, V8 b, f32x16& c) { c = mfma32_any(a, b, c); }
+template <int I, class V8> inline void pinned_s_mfma_first(V8 a, V8 b, f32x16& c) { c = mfma32_any(a, b, zero16()); }
+template <int I, class V8> inline void pinned_s_mfma(V8 a, V8 b, f32x16& c) { c = mfma32_any(a, b, c); }
+template <int I> inline void pinned_o_clear(f32x16& c) { c = zero16(); }
+template <int I> inline void pinned_o_scale(f32x16& c, float f) { for (int r = 0; r < 16; ++r) c[r] *= f; }
+template <int I, int R> inline float pinned_o_read(const f32x16& c) { return c[R]; }
+inline void mfma_drain() {}
+template <int R> inline float acc_read(const f32x16& c) { return c[R]; }
+template <int R> inline void acc_scale(f32x16& c, float f) { c[R] *= f; }
+template <int R> inline void acc_clear(f32x16& c) { c[R] = 0.f; }
 inline f32x16 mfma32_vacc(half8 a, half8 b, f32x16 c) { return mfma32_any(a, b, c); }
 inline f32x16 mfma32_vacc(bf16x8 a, bf16x8 b, f32x16 c) { return mfma32_any(a, b, c); }
 
@@ -261,6 +292,9 @@ inline short4v lds_read_tr16(const void* p) {
   return r;
 }
 
+inline u32x4 lds_load16(uint32_t addr) { return *(const u32x4*)(hwsim::lds + addr); }
+inline short4v lds_read_tr16_at(uint32_t addr) { return lds_read_tr16(hwsim::lds + addr); }
+
 inline float shfl_xor(float x, int mask) {
   hwsim::Lane& ln = hwsim::lanes[hwsim::cur];
   ln.sh_in = x;
@@ -269,6 +303,34 @@ inline float shfl_xor(float x, int mask) {
   return hwsim::lanes[hwsim::cur].sh_out;
 }
 inline float xor32(float x) { return shfl_xor(x, 32); }
+inline void swap_halves(float& a, float& b) {
+  const bool upper = (hwsim::cur & 63) >= 32;
+  const float xa = shfl_xor(a, 32), xb = shfl_xor(b, 32);
+  // a' = [a.lo, b.lo], b' = [a.hi, b.hi]
+  const float na = upper ? xb : a, nb = upper ? b : xa;
+  a = na;
+  b = nb;
+}
+inline float max3(float a, float b, float c) { return fmaxf(fmaxf(a, b), c); }
+inline float max2(float a, float b) { return fmaxf(a, b); }
+inline uint32_t lds_address(const void* p) { return (uint32_t)((const unsigned char*)p - hwsim::lds); }
+inline void dma_load16(const void* base, uint32_t lane_offset, uint32_t lds_base) {
+  memcpy(hwsim::lds + lds_base + 16 * (hwsim::cur & 63), (const char*)base + lane_offset, 16);
+}
+inline uint32_t pack2(half_t, float a, float b) {
+  half_t v[2] = {(half_t)a, (half_t)b};
+  uint32_t r; memcpy(&r, v, 4); return r;
+}
+inline uint32_t pack2(bf16_t, float a, float b) {
+  bf16_t v[2] = {(bf16_t)a, (bf16_t)b};
+  uint32_t r; memcpy(&r, v, 4); return r;
+}
+inline float add_pair(half_t, uint32_t pair, float acc) {
+  half_t v[2]; memcpy(v, &pair, 4); return acc + (float)v[0] + (float)v[1];
+}
+inline float add_pair(bf16_t, uint32_t pair, float acc) {
+  bf16_t v[2]; memcpy(v, &pair, 4); return acc + (float)v[0] + (float)v[1];
+}
 inline bool wave_any(bool pred) {
   float v = pred ? 1.f : 0.f;
   for (int m = 1; m < 64; m <<= 1) v = fmaxf(v, shfl_xor(v, m));
@@ -276,6 +338,8 @@ inline bool wave_any(bool pred) {
 }
 
 inline void sched_fence() {}
+inline void pin(float&) {}
+inline void pin(uint32_t&) {}
 template <class V> inline void keep_in_agprs(V&) {}
 inline void keep_branch() {}
 template <int N, int DEPTH, int RPM = 1, int EXTRA = 0> inline void sched_prefetched_operands() {}

@@ -81,6 +81,53 @@ def test_flash_forward_backward_total(lib, B, H, Hk, M, N, D, causal, dtype, bth
         assert torch.all(torch.isinf(lse[:, :, : M - N]))
 
 
+WIDE_CASES = [
+    # B, H, Hk, M, N, causal, dtype, bthd, std
+    (1, 1, 1, 64, 64, False, torch.bfloat16, False, 1.0),     # one tile
+    (1, 2, 1, 100, 150, True, torch.bfloat16, False, 1.0),    # grouped heads, ragged rows and keys
+    (1, 1, 1, 300, 300, True, torch.float16, True, 1.0),      # two row blocks, diagonal tiles, strided views
+    (1, 1, 1, 40, 1, False, torch.float16, False, 1.0),       # a single key
+    (1, 1, 1, 257, 520, True, torch.bfloat16, False, 1.0),    # steady loop, then masked tiles, then the last one
+    (1, 1, 1, 256, 640, False, torch.float16, False, 4.0),    # large late scores: the reference maximum is raised late
+    (1, 1, 1, 330, 130, True, torch.float16, False, 1.0),     # M > N: rows without keys
+]
+
+
+@pytest.mark.parametrize("B,H,Hk,M,N,causal,dtype,bthd,std", WIDE_CASES)
+def test_flash_forward_256_row_kernel(lib, B, H, Hk, M, N, causal, dtype, bthd, std):
+    """fa_fwd with block_m = 256: the slot-structured kernel with 64 query rows per wavefront (head
+    size 128), against the oracle and against the 128-row kernel."""
+    D = 128
+    q, k, v = rnd((B, H, M, D), dtype, bthd, std), rnd((B, Hk, N, D), dtype, bthd, std), rnd((B, Hk, N, D), dtype, bthd)
+    if std > 1:
+        k[..., N // 2:, :] *= 1.5
+    sc = 1 / math.sqrt(D)
+    o = torch.full_like(q, float("nan"))
+    lse = torch.full((B, H, M), float("nan"))
+    _abi.fa_fwd(lib, q, k, v, o, lse, causal, sc, block_m=256)
+    ref = flash_attention(q, k, v, causal, upcast=True, return_log_normalizer=True)
+    same = flash_attention(q, k, v, causal, upcast=False, return_log_normalizer=True)
+    check("o", o, same[0], ref[0])
+    check("lse", lse, same[1], ref[1])
+    o128, lse128 = torch.empty_like(o), torch.empty_like(lse)
+    _abi.fa_fwd(lib, q, k, v, o128, lse128, causal, sc, block_m=128)
+    assert torch.equal(torch.isinf(lse), torch.isinf(lse128))
+    fin = torch.isfinite(lse)
+    assert (lse[fin] - lse128[fin]).abs().max() < 1e-4
+    if causal and M > N:
+        assert torch.all(o[:, :, : M - N] == 0) and torch.all(torch.isinf(lse[:, :, : M - N]))
+
+
+def test_flash_forward_tile_argument_is_checked(lib):
+    q = rnd((1, 1, 64, 64), torch.float16)
+    o, lse = torch.empty_like(q), torch.empty(1, 1, 64)
+    with pytest.raises(AssertionError):   # the 256-row kernel exists for head size 128 only
+        _abi.fa_fwd(lib, q, q, q, o, lse, False, 0.125, block_m=256)
+    with pytest.raises(AssertionError):   # no such tile
+        _abi.fa_fwd(lib, q, q, q, o, lse, False, 0.125, block_m=64)
+    _abi.fa_fwd(lib, q, q, q, o, lse, False, 0.125, block_m=128)
+
+
 DS_CASES = [
     # B, H, Hk, M, N, D, causal, dtype, bthd
     (1, 2, 1, 100, 150, 128, True, torch.bfloat16, False),
