@@ -343,3 +343,58 @@ def test_ds_route_with_key_tail_and_very_negative_log_normalizer(M, N, causal, d
     same = torch.autograd.grad(oracle_flash(q, k, v, causal, upcast=False), (q, k, v), do)
     for name, h, s, r in zip(("dq", "dk", "dv"), (dq, dk, dv), same, ref):
         check(name, h, s, r)
+
+
+WIDE_SHAPES = [
+    # B, Hq, Hk, M, N  (head size 128)
+    (2, 4, 4, 512, 612), (2, 4, 2, 512, 612), (2, 4, 4, 4096, 4000), (2, 4, 2, 4096, 4001), (1, 2, 1, 4001, 4096),
+    (1, 8, 8, 2048, 2048), (1, 3, 1, 1000, 77), (2, 2, 2, 10006, 10), (1, 2, 2, 255, 8202), (1, 16, 4, 64, 64),
+]
+
+
+@pytest.mark.parametrize("scale", [1.0, 4.0])
+@pytest.mark.parametrize("B,Hq,Hk,M,N", WIDE_SHAPES)
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("order", ["BHTD", "BTHD"])
+def test_attention_fwd_256_row_kernel(B, Hq, Hk, M, N, causal, order, dtype, scale):
+    """The forward kernel with BLOCK_M = 256 (head size 128: 64 query rows per wavefront, slot-structured),
+    called through the C entry point with the tile named explicitly, under the same 2x rule for o and the
+    log-normalizer; rows without keys give o = 0 and -inf."""
+    from flagattention_amd import _abi, _lib
+    lib = _lib.get()
+    D = 128
+    q = make((B, Hq, M, D), dtype, order, scale, 1)
+    k = make((B, Hk, N, D), dtype, order, scale, 2)
+    v = make((B, Hk, N, D), dtype, order, scale, 3)
+    o = torch.full_like(q, float("nan"))
+    lse = torch.full((B, Hq, M), float("nan"), device="cuda")
+    _abi.fa_fwd(lib, q, k, v, o, lse, causal, D ** -0.5, block_m=256)
+    ref = oracle_flash(q, k, v, causal, upcast=True, return_log_normalizer=True)
+    same = oracle_flash(q, k, v, causal, upcast=False, return_log_normalizer=True)
+    check("o", o, same[0], ref[0])
+    check("log_normalizer", lse, same[1], ref[1])
+    if causal and M > N:
+        assert torch.all(o[:, :, : M - N] == 0) and torch.all(torch.isinf(lse[:, :, : M - N]))
+
+
+def test_forward_tile_hook_selects_the_kernel(monkeypatch):
+    """``flash.get_fwd_config`` chooses between the two compiled forward kernels (examples/use_cutom_config_func.py
+    of the reference): both answers give results within rounding of each other, and a tile that does not
+    apply to the launch falls back with a warning."""
+    import warnings
+    from flag_attn import flash
+    q, k, v = (make((1, 4, 1024, 128), torch.bfloat16, "BHTD", 1.0, s) for s in (1, 2, 3))
+    outs = {}
+    for bm in (128, 256):
+        monkeypatch.setattr(flash, "get_fwd_config", lambda B, H, M, N, D, causal, bm=bm: (bm, 64, 2, 4))
+        outs[bm] = flag_attn.flash_attention(q, k, v, causal=True, return_log_normalizer=True)
+    assert (outs[128][0].float() - outs[256][0].float()).abs().max() < 2e-2
+    assert (outs[128][1] - outs[256][1]).abs().max() < 1e-4
+    assert not torch.equal(outs[128][0], outs[256][0])   # two different kernels ran (summation order differs)
+    q64, k64, v64 = (make((1, 4, 1024, 64), torch.bfloat16, "BHTD", 1.0, s) for s in (1, 2, 3))
+    with warnings.catch_warnings(record=True) as seen:
+        warnings.simplefilter("always")
+        o = flag_attn.flash_attention(q64, k64, v64, causal=True)
+    check("o", o, oracle_flash(q64, k64, v64, True, upcast=False), oracle_flash(q64, k64, v64, True, upcast=True))
+    assert len(seen) <= 1
