@@ -223,6 +223,12 @@ FA_DEVICE short4v lds_read_tr16_at(uint32_t addr) {
 // True in every lane if the predicate holds in any lane of the wavefront.
 FA_DEVICE bool wave_any(bool pred) { return __builtin_amdgcn_ballot_w64(pred) != 0; }
 
+// Lanes of the wavefront in which the predicate holds, as a bit mask.
+FA_DEVICE uint64_t ballot(bool pred) { return __builtin_amdgcn_ballot_w64(pred); }
+// Value held by lane l - delta (lanes below delta keep their own), and by a given lane.
+FA_DEVICE int shfl_up(int x, int delta) { return __shfl_up(x, delta, 64); }
+FA_DEVICE int lane_value(int x, int lane) { return __shfl(x, lane, 64); }
+
 // Value held by lane (l ^ 32).
 FA_DEVICE float xor32(float x) { return __shfl_xor(x, 32, 64); }
 // Value held by lane (l ^ mask) for mask < 64.

@@ -194,31 +194,27 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (D <= 128 ? 2 : 1)) paged_balanced_ke
   const int pairs_per_seq = p.Hkv * row_blocks;
   auto units_of = [&](int seq) { const int c = p.context_lens[seq]; return c > 0 ? (c + kUnitKeys - 1) / kUnitKeys : 0; };
 
-  // ---- every workgroup scans the context lengths (num_seqs values, served from L2) ----
-  const int chunk = cdiv(p.num_seqs, kThreads);
-  const int s_lo = imin(p.num_seqs, tid * chunk), s_hi = imin(p.num_seqs, s_lo + chunk);
-  int mine = 0;
-  for (int s = s_lo; s < s_hi; ++s) {
-    const int u = units_of(s);
-    mine += u;
-    if (u == 0 && w == 0) {  // an empty sequence has no keys to stream: its output rows are zero
+  // ---- every wavefront scans the context lengths for itself, 64 at a time: no LDS, no barrier ----
+  auto prefix_in_wave = [&](int u) {   // inclusive prefix sum over the lanes
+    int incl = u;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int t = hw::shfl_up(incl, d);
+      if (lane >= d) incl += t;
+    }
+    return incl;
+  };
+  int total_units = 0;
+  for (int base = 0; base < p.num_seqs; base += 64) {
+    const int s = base + lane;
+    const int u = s < p.num_seqs ? units_of(s) : 0;
+    if (w == 0 && tid < 64 && s < p.num_seqs && u == 0) {  // an empty sequence has no keys to stream: its output rows are zero
       for (int i = 0; i < p.Hq * D; ++i) ((T*)p.out)[(int64_t)s * p.o_ss + (int64_t)(i / D) * p.o_sh + i % D] = (T)0.f;
     }
+    total_units += hw::uniform(hw::lane_value(prefix_in_wave(u), 63));
   }
-  int* scan_a = (int*)smem;
-  int* scan_b = scan_a + kThreads;
-  int* found = scan_b + kThreads;  // {first sequence of this workgroup, units before it}
-  scan_a[tid] = mine;
-  hw::block_sync();
-  for (int off = 1; off < kThreads; off <<= 1) {
-    const int v = scan_a[tid] + (tid >= off ? scan_a[tid - off] : 0);
-    scan_b[tid] = v;
-    hw::block_sync();
-    int* t = scan_a; scan_a = scan_b; scan_b = t;
-  }
-  // read through a scalar register: everything derived from it (the key ranges, the step counts of
-  // the wavefronts) then stays in scalar registers too
-  const int64_t total = (int64_t)hw::uniform(scan_a[kThreads - 1]) * pairs_per_seq;
+  // everything derived from the total (the key ranges, the step counts of the wavefronts) stays in scalar registers
+  const int64_t total = (int64_t)total_units * pairs_per_seq;
   const int64_t per = (int64_t)imax(kMinUnitsPerWg, (int)((total + p.num_wgs - 1) / p.num_wgs));
   const int64_t u_begin = (int64_t)w * per;
   const int64_t u_end = u_begin + per < total ? u_begin + per : total;
@@ -227,20 +223,25 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (D <= 128 ? 2 : 1)) paged_balanced_ke
     if (tid == 0) meta[3] = 0;
     return;
   }
+  // the sequence whose pairs hold unit u_begin, and the units of the sequences before it
+  int seq = 0, before = 0;
   {
-    const int incl = scan_a[tid], excl = incl - mine;
-    if ((int64_t)excl * pairs_per_seq <= u_begin && u_begin < (int64_t)incl * pairs_per_seq) {
-      int pre = excl;
-      for (int s = s_lo; s < s_hi; ++s) {
-        const int u = units_of(s);
-        if (u_begin < (int64_t)(pre + u) * pairs_per_seq) { found[0] = s; found[1] = pre; break; }
-        pre += u;
-      }
+    int running = 0;
+    for (int base = 0; base < p.num_seqs; base += 64) {
+      const int s = base + lane;
+      const int u = s < p.num_seqs ? units_of(s) : 0;
+      const int incl = prefix_in_wave(u), excl = incl - u;
+      const bool here = u > 0 && (int64_t)(running + excl) * pairs_per_seq <= u_begin &&
+                        u_begin < (int64_t)(running + incl) * pairs_per_seq;
+      const uint64_t hit = hw::ballot(here);
+      const int first = hit ? __builtin_ctzll(hit) : 0;
+      const int excl_first = hw::lane_value(excl, first), all = hw::lane_value(incl, 63);
+      if (hit) { seq = base + first; before = running + excl_first; }
+      running += all;
     }
+    seq = hw::uniform(seq);
+    before = hw::uniform(before);
   }
-  hw::block_sync();
-  int seq = hw::uniform(found[0]);
-  int before = hw::uniform(found[1]);
   int64_t u = u_begin;
   int unfinished = 0;
 
@@ -259,7 +260,7 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (D <= 128 ? 2 : 1)) paged_balanced_ke
     const T* q_row = nullptr;
     if (g_lane < G) q_row = (const T*)p.q + (int64_t)seq * p.q_ss + (int64_t)(hk * G + g_lane) * p.q_sh;
 
-    hw::block_sync();  // the scan, or the previous pair's merge area, is read out before staging reuses it
+    hw::block_sync();  // the previous pair's merge area is read out before staging reuses it
     DecodeOut<D> res;
     decode_block<T, D>(src, q_row, n_begin, n_end, n_end, p.scale * kLog2e, smem, res);
 

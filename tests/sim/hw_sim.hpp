@@ -303,6 +303,35 @@ inline float shfl_xor(float x, int mask) {
   return hwsim::lanes[hwsim::cur].sh_out;
 }
 inline float xor32(float x) { return shfl_xor(x, 32); }
+// integer exchanges ride on the float one (values are small enough to be exact)
+inline int shfl_up(int x, int delta) {
+  // value of lane l - delta: gather through xor exchanges of every source lane bit pattern
+  int result = x;
+  const int me = hwsim::cur & 63;
+  for (int m = 1; m < 64; ++m) {
+    const int got = (int)shfl_xor((float)x, m);
+    if ((me ^ m) == me - delta) result = got;
+  }
+  return result;
+}
+inline int lane_value(int x, int lane) {
+  int result = x;
+  const int me = hwsim::cur & 63;
+  for (int m = 1; m < 64; ++m) {
+    const int got = (int)shfl_xor((float)x, m);
+    if ((me ^ m) == lane) result = got;
+  }
+  return result;
+}
+inline uint64_t ballot(bool pred) {
+  uint64_t mask = 0;
+  const int me = hwsim::cur & 63;
+  for (int m = 0; m < 64; ++m) {
+    const float got = m == 0 ? (pred ? 1.f : 0.f) : shfl_xor(pred ? 1.f : 0.f, m);
+    if (got > 0.f) mask |= (uint64_t)1 << (me ^ m);
+  }
+  return mask;
+}
 inline void swap_halves(float& a, float& b) {
   const bool upper = (hwsim::cur & 63) >= 32;
   const float xa = shfl_xor(a, 32), xb = shfl_xor(b, 32);
