@@ -53,19 +53,43 @@ def causal_pairs(M, N):
     return sum(min(max(m + N - M + 1, 0), N) for m in range(M))
 
 
-def timed_launches(fn, iters, torch):
-    """Mean duration in ms of ``fn`` over ``iters`` launches, HIP events on the current stream."""
+def timed_launches(fn, iters, torch, groups=5):
+    """Duration in ms of one ``fn``: the median over ``groups`` groups of the mean of ``iters``
+    back-to-back launches, each group bracketed by HIP events on the current stream (the stream the
+    C entry points launch on)."""
     for _ in range(3):
         fn()
-    start = torch.cuda.Event(enable_timing=True)
-    stop = torch.cuda.Event(enable_timing=True)
-    torch.cuda.synchronize()
-    start.record()
-    for _ in range(iters):
-        fn()
-    stop.record()
-    stop.synchronize()
-    return start.elapsed_time(stop) / iters
+    means = []
+    for _ in range(groups):
+        start = torch.cuda.Event(enable_timing=True)
+        stop = torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        start.record()
+        for _ in range(iters):
+            fn()
+        stop.record()
+        stop.synchronize()
+        means.append(start.elapsed_time(stop) / iters)
+    means.sort()
+    return means[len(means) // 2]
+
+
+def flash_step_leg(torch, B, H, Tq, Tk, D, iters=5):
+    """One more flash_attention forward + backward configuration, public API, as a small record."""
+    import flagattention_amd as flag_attn
+    dev = "cuda:0"
+    g = torch.Generator(device=dev).manual_seed(10086)
+    mk = lambda T: torch.randn(B, H, T, D, device=dev, dtype=torch.bfloat16, generator=g)
+    q, k, v, do = mk(Tq).requires_grad_(), mk(Tk).requires_grad_(), mk(Tk).requires_grad_(), mk(Tq)
+    sm_scale = 1.0 / math.sqrt(D)
+    ms_fwd = timed_launches(lambda: flag_attn.flash_attention(q, k, v, causal=True, sm_scale=sm_scale), iters, torch)
+    o = flag_attn.flash_attention(q, k, v, causal=True, sm_scale=sm_scale)
+    ms_bwd = timed_launches(lambda: torch.autograd.grad(o, (q, k, v), do, retain_graph=True), iters, torch)
+    flop = 7 * 2.0 * B * H * causal_pairs(Tq, Tk) * D
+    tf = flop / ((ms_fwd + ms_bwd) * 1e-3) / 1e12
+    return {"workload": f"flash_attention fwd+bwd causal bf16 B={B} H={H} Tq={Tq} Tk={Tk} D={D}",
+            "ms_fwd": round(ms_fwd, 4), "ms_bwd": round(ms_bwd, 4), "counted_gflop": round(flop / 1e9, 2),
+            "value": round(tf, 1), "unit": "TFLOP/s", "frac_of_mfma_peak": round(tf / PEAK_BF16_TFLOPS, 4)}
 
 
 def flash_step_bench(args, torch):
@@ -171,7 +195,7 @@ def cpu_baseline(args, torch):
                       f"fwd+bwd, best of 2, {best:.2f} s"}
 
 
-def paged_bench(torch, iters=50):
+def paged_bench(torch, iters=50, groups=5):
     import flagattention_amd as flag_attn
     dev = "cuda:0"
     g = torch.Generator(device=dev).manual_seed(10086)
@@ -192,7 +216,7 @@ def paged_bench(torch, iters=50):
     vc = torch.randn(num_blocks, Hkv, bs, D, device=dev, dtype=torch.float16, generator=g)
     scale = D ** -0.5
     fn = lambda: flag_attn.paged_attention(q, kc, vc, ctx, bt, scale, max_ctx)
-    ms = timed_launches(fn, iters, torch)
+    ms = timed_launches(fn, iters, torch, groups)
     total_ctx = int(ctx.sum().item())
     kv_bytes = total_ctx * Hkv * D * 2 * 2
     algo = kv_bytes + 2 * q.numel() * 2 + 8 * num_blocks
@@ -203,25 +227,36 @@ def paged_bench(torch, iters=50):
                          "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": PAGED_TRAFFIC_BYTES}}
 
 
-def splitkv_bench(torch, iters=50):
+def splitkv_bench(torch, iters=48, groups=5, sets=3):
     """Dense split-KV decode through flash_attention: q (4, 32, 1, 128), k/v (4, 8, 32768, 128) fp16."""
     import flagattention_amd as flag_attn
     dev = "cuda:0"
     g = torch.Generator(device=dev).manual_seed(10086)
     B, H, Hk, N, D = 4, 32, 8, 32768, 128
     q = torch.randn(B, H, 1, D, device=dev, dtype=torch.float16, generator=g)
-    k = torch.randn(B, Hk, N, D, device=dev, dtype=torch.float16, generator=g)
-    v = torch.randn(B, Hk, N, D, device=dev, dtype=torch.float16, generator=g)
-    ms = timed_launches(lambda: flag_attn.flash_attention(q, k, v, causal=False), iters, torch)
+    # Three distinct K/V sets (3 x 537 MB) used in turn: a launch never finds its keys and values in
+    # the 256 MB last-level cache left there by the launch before it.
+    sets = [(torch.randn(B, Hk, N, D, device=dev, dtype=torch.float16, generator=g),
+             torch.randn(B, Hk, N, D, device=dev, dtype=torch.float16, generator=g)) for _ in range(sets)]
+    turn = [0]
+
+    def launch():
+        k, v = sets[turn[0] % len(sets)]
+        turn[0] += 1
+        return flag_attn.flash_attention(q, k, v, causal=False)
+
+    ms = timed_launches(launch, iters, torch, groups)
+    k = sets[0][0]
     algo = 2 * k.numel() * 2 + 2 * q.numel() * 2
     gbs = algo / (ms * 1e-3) / 1e9
-    return {"workload": "flash_attention decode fp16 q=(4,32,1,128) k/v=(4,8,32768,128) (split-KV path)",
+    return {"workload": "flash_attention decode fp16 q=(4,32,1,128) k/v=(4,8,32768,128) (split-KV path), "
+                        f"{len(sets)} K/V sets in rotation",
             "ms": round(ms, 4), "algorithmic_bytes": algo, "value": round(gbs, 1), "unit": "GB/s",
             "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                          "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None}}
 
 
-def piecewise_bench(torch, iters=10):
+def piecewise_bench(torch, iters=10, groups=5):
     """piecewise_attention forward + backward, causal bf16 B=2 H=32 T=4096 D=128, threshold 1024.
     FLOPs counted as for flash attention (one dot product per score), not with the reference's
     1.5x / 1.6x convention for its two score products (benchmark/piecewise_benchmark.py:98-110)."""
@@ -231,9 +266,9 @@ def piecewise_bench(torch, iters=10):
     B, H, T, D, w = 2, 32, 4096, 128, 1024
     ts = [torch.randn(B, H, T, D, device=dev, dtype=torch.bfloat16, generator=g).requires_grad_() for _ in range(5)]
     do = torch.randn(B, H, T, D, device=dev, dtype=torch.bfloat16, generator=g)
-    ms_fwd = timed_launches(lambda: flag_attn.piecewise_attention(*ts, w, causal=True), iters, torch)
+    ms_fwd = timed_launches(lambda: flag_attn.piecewise_attention(*ts, w, causal=True), iters, torch, groups)
     o = flag_attn.piecewise_attention(*ts, w, causal=True)
-    ms_bwd = timed_launches(lambda: torch.autograd.grad(o, ts, do, retain_graph=True), iters, torch)
+    ms_bwd = timed_launches(lambda: torch.autograd.grad(o, ts, do, retain_graph=True), iters, torch, groups)
     fwd = 4.0 * B * H * causal_pairs(T, T) * D
     tf = (fwd * 3.5) / ((ms_fwd + ms_bwd) * 1e-3) / 1e12
     return {"workload": "piecewise_attention fwd+bwd causal bf16 B=2 H=32 T=4096 D=128 dist_threshold=1024",
@@ -243,7 +278,7 @@ def piecewise_bench(torch, iters=10):
                          "frac": round(tf / PEAK_BF16_TFLOPS, 4), "traffic": None}}
 
 
-def total_attention_bench(torch, iters=20):
+def total_attention_bench(torch, iters=20, groups=5):
     """total_attention (column sums of P) at the benchmark shape: one product, 2 * pairs * D per head."""
     import flagattention_amd as flag_attn
     dev = "cuda:0"
@@ -251,7 +286,7 @@ def total_attention_bench(torch, iters=20):
     B, H, T, D = 1, 32, 8192, 128
     q, k, v = (torch.randn(B, H, T, D, device=dev, dtype=torch.bfloat16, generator=g) for _ in range(3))
     _, L, _, _, _ = flag_attn.flash_attention(q, k, v, causal=True, return_log_normalizer=True)
-    ms = timed_launches(lambda: flag_attn.total_attention(q, k, L, True, D ** -0.5), iters, torch)
+    ms = timed_launches(lambda: flag_attn.total_attention(q, k, L, True, D ** -0.5), iters, torch, groups)
     flop = 2.0 * B * H * causal_pairs(T, T) * D
     tf = flop / (ms * 1e-3) / 1e12
     return {"workload": "total_attention causal bf16 B=1 H=32 T=8192 D=128", "ms": round(ms, 4),
@@ -273,8 +308,12 @@ def profile_kernel(args, torch):
         torch.cuda.synchronize()
         print(json.dumps({"profiled": "copy", "bytes_read": 1 << 30, "bytes_written": 1 << 30}))
         return
-    if args.profile_kernel == "paged_attn":
-        print(json.dumps({"profiled": "paged_attn", **paged_bench(torch, iters=5)}))
+    whole_legs = {"paged_attn": lambda: paged_bench(torch, iters=2, groups=1),
+                  "splitkv": lambda: splitkv_bench(torch, iters=3, groups=1),
+                  "piecewise": lambda: piecewise_bench(torch, iters=2, groups=1),
+                  "total_attention": lambda: total_attention_bench(torch, iters=2, groups=1)}
+    if args.profile_kernel in whole_legs:
+        print(json.dumps({"profiled": args.profile_kernel, **whole_legs[args.profile_kernel]()}))
         return
     w = WORKLOADS[args.workload]
     B, H, T, D = w["B"], w["H"], w["T"], w["D"]
@@ -315,7 +354,7 @@ def main():
     ap.add_argument("--workload", choices=sorted(WORKLOADS), default="c3")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--profile-kernel", choices=["fa_fwd", "fa_bwd_dkdv", "fa_bwd_dkdv_ds", "fa_bwd_dq", "fa_bwd_dq_from_ds",
-                                                  "paged_attn", "copy"],
+                                                  "paged_attn", "splitkv", "piecewise", "total_attention", "copy"],
                     help="run only this launch a few times (for rocprofv3 counter passes); 'copy' is a plain "
                          "1 GiB device copy used to calibrate FETCH_SIZE / WRITE_SIZE")
     ap.add_argument("--hold-seconds", type=float, default=0.0,
@@ -344,6 +383,11 @@ def main():
         "kernels": kernels,
     }
     if not args.no_paged:
+        # The other flash configurations of the workload list, as records of their own.
+        legs = {"c2": (4, 16, 2048, 2048, 128), "c3": (1, 32, 8192, 8192, 128),
+                "c3_d64": (1, 32, 8192, 8192, 64), "cross_length": (1, 32, 1024, 8192, 128)}
+        legs.pop(args.workload, None)
+        out["other_flash_workloads"] = {name: flash_step_leg(torch, *shape) for name, shape in legs.items()}
         out["paged_decode"] = paged_bench(torch)
         out["splitkv_decode"] = splitkv_bench(torch)
         out["piecewise"] = piecewise_bench(torch)

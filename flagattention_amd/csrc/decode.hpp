@@ -5,9 +5,10 @@
 //   * a workgroup serves up to 16 query rows that share one key/value head (all query heads of a
 //     GQA group, times the few query positions), so K and V are read once per kv head;
 //   * the products use the 16x16x32 MFMA: with 16 query rows the output accumulator O^T (D x 16)
-//     needs D/4 registers and the scores of a 32-key step 8, which leaves room for TWO register sets
-//     of key/value loads -- while one 32-key step is computed the loads of the next two are in flight
-//     (32 KB per wavefront at D = 128, 256 KB per CU with two wavefronts per SIMD);
+//     needs D/4 registers and the scores of a 32-key step 8, which leaves room for a register set
+//     of key/value loads -- while one 32-key step is computed the loads of the next one are in
+//     flight (NSETS = 1: 16 KB per wavefront at D = 128, 128 KB per CU with two wavefronts per
+//     SIMD; the code also carries a second set, NSETS = 2, which is not switched on);
 //   * each of the 4 wavefronts walks its own interleaved sequence of 32-key steps with no workgroup
 //     barrier inside the loop: coalesced 16-byte global loads into registers, a private LDS patch to
 //     re-layout them, S^T = K Q^T (keys x queries, one query row per lane of each 16-lane group) and

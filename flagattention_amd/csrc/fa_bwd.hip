@@ -269,7 +269,23 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
     // commits its successor to LDS and then requests the tile after that
     if (t_begin + 1 < t_end) fetch((t_begin + 1) * C::BM);
 
-    for (int it = t_begin; it < t_end; ++it) {
+    // Does no mask touch the tile, so that it can run the slot-structured body?  (The same answer in
+    // every lane of a wavefront: read through a scalar register so that the loops below branch on it.)
+    auto is_plain = [&](int it) {
+      if constexpr (!FOLDED) return false;
+      const int m0 = it * C::BM;
+      // a block with keys past N goes through the masked path: its P and dS must be exact zeroes
+      // there (K and V rows are zero, so the score is just -L and exp2 of it can be huge)
+      bool plain = (nw + 31 < N) && (!p.causal || (m0 + pseq >= nw + 31));
+      // piecewise: every entry of the 64 x 32 tile belongs to this pass's regime
+      if (PW) plain = plain && (far_phase ? (m0 + pseq - (nw + 31) >= p.w) : (m0 + 63 + pseq - nw < p.w));
+      return hw::uniform((int)plain) != 0;
+    };
+    // One query tile.  The two bodies are separate instantiations, run from loops of their own (below): with
+    // both inside one loop the compiler carries the flags that tell them apart through every iteration and
+    // allocates registers for the union of the two.
+    auto tile = [&](auto plain_tag, int it) {
+      constexpr bool plain_tile = decltype(plain_tag)::value;
       const int m0 = it * C::BM;
       const bool more = it + 1 < t_end;
 
@@ -279,7 +295,7 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
       const float* sL = (const float*)(base + 2 * C::TILE * sizeof(T));
       const float* sDl = sL + C::BM;
       const int next_stage = stage + 1 == C::STAGES ? 0 : stage + 1;
-      bool committed_in_slots = false, synced_in_slots = false, fetched_in_slots = false;
+      constexpr bool committed_in_slots = plain_tile, synced_in_slots = plain_tile, fetched_in_slots = plain_tile;
 
       // Tiles that no mask touches (all but the one or two on the diagonal), with one wavefront per
       // SIMD: nothing else would issue under this wavefront's matrix instructions, so the
@@ -287,16 +303,8 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
       // other, one element per matrix instruction, in the order
       //   A0 | A1 with E0 | C0 with E1 | C1      (A: S and dP, E: P and dS, C: dV and dK)
       // and a scheduling fence after every such slot keeps the compiler from regrouping them.
-      bool plain_tile = false;
-      if constexpr (FOLDED) {
-        // a block with keys past N goes through the masked path: its P and dS must be exact zeroes
-        // there (K and V rows are zero, so the score is just -L and exp2 of it can be huge)
-        plain_tile = (nw + 31 < N) && (!p.causal || (m0 + pseq >= nw + 31));
-        // piecewise: every entry of the 64 x 32 tile belongs to this pass's regime
-        if (PW) plain_tile = plain_tile && (far_phase ? (m0 + pseq - (nw + 31) >= p.w) : (m0 + 63 + pseq - nw < p.w));
-      }
-      if constexpr (FOLDED) {
-      if (plain_tile) {
+      if constexpr (plain_tile) {
+      {
         constexpr int NA = 2 * C::KSTEPS;       // matrix instructions of an A phase (16)
         constexpr int NC = 4 * (C::DV / 32);    // of a C phase (16)
         static_assert(NA == 16 && NC == 16, "one element of a block per matrix instruction");
@@ -396,7 +404,6 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
         const int m_ahead = imin(it + 2, t_end - 1) * C::BM;
         const T* q_ahead = q_src + (int64_t)m_ahead * q_stride;
         const T* g_ahead = gb + (int64_t)m_ahead * p.dout.st;
-        committed_in_slots = synced_in_slots = fetched_in_slots = true;
         T* nQ = (T*)(smem + next_stage * C::STAGE_BYTES);
         T* nG = nQ + C::TILE;
         float* nf = (float*)(nG + C::TILE);
@@ -446,7 +453,7 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
         });
       }
       }
-      if (!plain_tile) {
+      if constexpr (!plain_tile) {
 #pragma unroll
       for (int sb = 0; sb < C::BM / 32; ++sb) {
         const int mr0 = m0 + sb * 32;
@@ -524,10 +531,21 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
       }
       }
 
-      if (more && !committed_in_slots) commit(next_stage);
-      if (!synced_in_slots) hw::block_sync();
-      if (!fetched_in_slots && it + 2 < t_end) fetch(m0 + 2 * C::BM);
+      if constexpr (!committed_in_slots) { if (more) commit(next_stage); }
+      if constexpr (!synced_in_slots) hw::block_sync();
+      if constexpr (!fetched_in_slots) { if (it + 2 < t_end) fetch(m0 + 2 * C::BM); }
       stage = next_stage;
+    };
+    {
+      int it = t_begin;
+      while (it < t_end) {
+        if constexpr (FOLDED) {
+#pragma unroll 1
+          for (; it < t_end && is_plain(it); ++it) tile(std::true_type{}, it);
+        }
+#pragma unroll 1
+        for (; it < t_end && !is_plain(it); ++it) tile(std::false_type{}, it);
+      }
     }
 
     if (PW) {  // this regime's dK is complete (piecewise has no grouped heads)

@@ -24,8 +24,8 @@ def randn(shape, dtype, seed, grad=False):
     return t.requires_grad_() if grad else t
 
 
-def check(name, hyp, same, ref):
-    ok, e_hyp, e_same = within_two_x(hyp, same, ref)
+def check(name, hyp, same, ref, strict=False):
+    ok, e_hyp, e_same = within_two_x(hyp, same, ref, strict=strict)
     assert ok, f"{name}: hip err {e_hyp:.3e} vs same-precision torch err {e_same:.3e}"
 
 
@@ -58,7 +58,7 @@ def _flash_fwd_bwd_case(B, H, M, N, D, head_slice=None):
     check("L", L[:, hs], same[1], ref[1])
     check("total", tot[:, hs], same[2], ref[2])
     for name, h, s, r in zip(("dq", "dk", "dv"), grads, g_same, g_ref):
-        check(name, h[:, hs], s, r)
+        check(name, h[:, hs], s, r, strict=True)   # "<" as in test_flash_attention.py:174-177 of the reference
 
 
 def test_c2_forward_backward_causal_bf16():

@@ -60,8 +60,8 @@ def make(shape, dtype, order, std, seed, grad=False):
     return t.requires_grad_() if grad else t
 
 
-def check(name, hyp, same, ref):
-    ok, e_hyp, e_same = within_two_x(hyp, same, ref)
+def check(name, hyp, same, ref, strict=False):
+    ok, e_hyp, e_same = within_two_x(hyp, same, ref, strict=strict)
     assert ok, f"{name}: hip err {e_hyp:.3e} vs same-precision torch err {e_same:.3e}"
 
 
@@ -112,10 +112,11 @@ def test_attention_bwd(B, Hq, Hk, M, N, D, causal, order, dtype, scale):
     g_ref = torch.autograd.grad(o_ref, (q, k, v), do)
     g_same = torch.autograd.grad(o_same, (q, k, v), do)
     g_hyp = torch.autograd.grad(o_hyp, (q, k, v), do)
-    check("o", o_hyp, o_same, o_ref)
+    # strict "<", as the reference's backward tests compare (test_flash_attention.py:174-177, 317-320)
+    check("o", o_hyp, o_same, o_ref, strict=True)
     for name, h, s, r in zip(("dq", "dk", "dv"), g_hyp, g_same, g_ref):
         assert h.shape == r.shape
-        check(name, h, s, r)
+        check(name, h, s, r, strict=True)
 
 
 @pytest.mark.parametrize("scale", [1.0, 2.0, 3.0, 4.0])
