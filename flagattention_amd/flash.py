@@ -147,18 +147,21 @@ class FlashAttention(torch.autograd.Function):
             dv = torch.empty((B, slices, N, D), dtype=v.dtype, device=q.device)
             dq = torch.empty((B, H, M, D), dtype=q.dtype, device=q.device)
             heads = ds_heads_per_launch(lib, B, H, group, M, N, D)
-            if heads == 0:
+            ds = None
+            if heads >= B * H:
+                ds = _ds_workspace(lib, q.device, B, H, M, N)
+            elif heads > 0:
+                heads = min(heads, H)
+                ds = _ds_workspace(lib, q.device, 1, heads, M, N)
+            if ds is None:   # dS not worth keeping for this shape, or no memory for it: recompute it
                 _abi.fa_bwd_dkdv(lib, q, k, v, do, L, delta, dk, dv, causal, sm_scale, dropout)
                 _abi.fa_bwd_dq(lib, q, k, v, do, L, delta, dq, causal, sm_scale, dropout)
             elif heads >= B * H:
-                ds = _ds_workspace(lib, q.device, B, H, M, N)
                 _abi.fa_bwd_dkdv_ds(lib, q, k, v, do, L, delta, dk, dv, ds, causal, sm_scale, dropout)
                 _abi.fa_bwd_dq_from_ds(lib, k, ds, dq, causal, sm_scale)
             else:
                 # bounded workspace: one batch entry and `heads` query heads at a time; the dropout
                 # counter of a slice starts where the slice starts in the (B, H, M, N) score tensor
-                heads = min(heads, H)
-                ds = _ds_workspace(lib, q.device, 1, heads, M, N)
                 for b in range(B):
                     for h0 in range(0, H, heads):
                         h1 = min(H, h0 + heads)
@@ -189,8 +192,14 @@ def dkdv_heads_per_slice(B, H, group, N, num_cus):
     return 1
 
 
-# Largest dS workspace the backward may take (MiB); 0 disables the dS path.
-DS_WORKSPACE_LIMIT_MIB = int(os.environ.get("FLAGATTN_DS_WORKSPACE_MIB", "8192"))
+# Largest dS workspace the backward may take (MiB); 0 disables the dS path.  The workspace is
+# M * N * 2 bytes per (batch, head) slice (128 MiB at 8192 x 8192); a backward whose slices do not
+# all fit walks them in launches of as many heads as do.  Launches of fewer than about 32 heads of
+# 8192 keys no longer fill the device: measured at B = 1, H = 32, T = 8192, D = 128 (needs 4096 MiB),
+# a forward + backward step takes 2.16 ms with 4096 MiB or more, 2.20 with 2048, 2.33 with 1024,
+# 3.11 with 512 and 5.51 with 256.  The default holds that workload whole.  A workspace that cannot be
+# allocated is not an error: the backward then recomputes dS (the fa_bwd_dkdv + fa_bwd_dq pair).
+DS_WORKSPACE_LIMIT_MIB = int(os.environ.get("FLAGATTN_DS_WORKSPACE_MIB", "4096"))
 
 
 def ds_heads_per_launch(lib, B, H, group, M, N, D, grids=1):
@@ -210,9 +219,13 @@ def ds_heads_per_launch(lib, B, H, group, M, N, D, grids=1):
 
 
 def _ds_workspace(lib, device, B, H, M, N, grids=1):
+    """Device memory for dS, or None when the allocator has none left (the caller then recomputes)."""
     mib = lib.fa_bwd_ds_workspace_mib(B, H, M, N)
     assert mib > 0
-    return torch.empty(grids * (mib << 20), dtype=torch.uint8, device=device)
+    try:
+        return torch.empty(grids * (mib << 20), dtype=torch.uint8, device=device)
+    except torch.OutOfMemoryError:
+        return None
 
 
 def attention(q, k, v, causal=False, sm_scale=None, dropout_p=0.0,

@@ -72,16 +72,19 @@ class PiecewiseAttention(torch.autograd.Function):
             args = (ctx.w, ctx.causal, ctx.sm_scale)
             # dS handed from the dK/dV kernel to the dQ kernels, one chunk grid per regime, when it pays
             heads = ds_heads_per_launch(lib, B, H, 1, M, N, D, grids=2)
-            if heads == 0:
+            ds = None
+            if heads >= B * H:
+                ds = _ds_workspace(lib, q1.device, B, H, M, N, grids=2)
+            elif heads > 0:
+                heads = min(heads, H)
+                ds = _ds_workspace(lib, q1.device, 1, heads, M, N, grids=2)
+            if ds is None:   # dS not worth keeping for this shape, or no memory for it: recompute it
                 _abi.pw_bwd_dkdv(lib, q1, k1, q2, k2, v, do, L, delta, dk1, dk2, dv, *args)
                 _abi.pw_bwd_dq(lib, q1, k1, q2, k2, v, do, L, delta, dq1, dq2, *args)
             elif heads >= B * H:
-                ds = _ds_workspace(lib, q1.device, B, H, M, N, grids=2)
                 _abi.pw_bwd_dkdv_ds(lib, q1, k1, q2, k2, v, do, L, delta, dk1, dk2, dv, ds, *args)
                 _abi.pw_bwd_dq_from_ds(lib, k1, k2, ds, dq1, dq2, *args)
             else:  # bounded workspace: one batch entry and `heads` heads at a time
-                heads = min(heads, H)
-                ds = _ds_workspace(lib, q1.device, 1, heads, M, N, grids=2)
                 for b in range(B):
                     for h0 in range(0, H, heads):
                         s = (slice(b, b + 1), slice(h0, min(H, h0 + heads)))

@@ -94,8 +94,12 @@ int fa_bwd_dq(int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v
  * fa_bwd_dq_from_ds computes dq = sm_scale * dS k from it -- one matrix product instead of three,
  * for one write and one read of a (B, H, M, N) matrix.  The workspace is device memory of at least
  * fa_bwd_ds_workspace_mib(B, H, M, N) MiB, 16-byte aligned, in a private blocked order; its contents
- * on entry do not matter.  Both calls must use the same B, H, M, N and causal flag; to bound the
- * workspace, callers may process slices of the batch or of the heads one after the other. */
+ * on entry do not matter.  Its size grows with the score matrix, O(M * N) per (batch, head) slice:
+ * B * H * ceil(M / 128) * ceil(N / 128) * 32 KiB, i.e. 2 bytes per score with M and N rounded up to
+ * 128 (128 MiB per slice at M = N = 8192, 4 GiB for 32 such slices), whether or not the mask is
+ * causal.  Both calls must use the same B, H, M, N and causal flag; to bound the workspace, callers
+ * may process slices of the batch or of the heads one after the other, with launches of at least
+ * about 32 heads x 8192 keys if the device is to stay full. */
 int fa_bwd_ds_workspace_mib(int B, int H, int M, int N);
 int fa_bwd_dkdv_ds(int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v,
                    const fa_view4* dout, const float* lse, const float* delta, const fa_view4* dk,

@@ -150,3 +150,38 @@ def test_default_hooks_name_compiled_tiles():
     for mod in (flash, piecewise):
         assert mod.get_fwd_config(1, 1, 4096, 4096, 128, True)[:2] in mod.FWD_TILES
         assert mod.get_bwd_config(1, 1, 4096, 4096, 128, True)[:2] in mod.BWD_TILES
+
+
+class _SizesOnly:
+    """Stands in for the kernel library where only the workspace size is asked for."""
+
+    @staticmethod
+    def fa_bwd_ds_workspace_mib(B, H, M, N):
+        return (B * H * -(-M // 128) * -(-N // 128) * 32768 + (1 << 20) - 1) >> 20
+
+
+def test_ds_workspace_policy(monkeypatch):
+    from flagattention_amd import flash
+    lib = _SizesOnly()
+    monkeypatch.setattr(flash, "DS_WORKSPACE_LIMIT_MIB", 4096)
+    # the headline shape needs 32 x 128 MiB and is held whole; twice the batch goes in slices
+    assert flash.ds_heads_per_launch(lib, 1, 32, 1, 8192, 8192, 128) == 32
+    assert flash.ds_heads_per_launch(lib, 2, 32, 1, 8192, 8192, 128) == 32
+    # slices are whole groups of query heads
+    monkeypatch.setattr(flash, "DS_WORKSPACE_LIMIT_MIB", 128 * 7)
+    assert flash.ds_heads_per_launch(lib, 1, 32, 4, 8192, 8192, 128) == 4
+    # small matrices, small heads and a zero limit recompute dS
+    assert flash.ds_heads_per_launch(lib, 1, 32, 1, 512, 512, 128) == 0
+    assert flash.ds_heads_per_launch(lib, 1, 32, 1, 8192, 8192, 64) == 0
+    monkeypatch.setattr(flash, "DS_WORKSPACE_LIMIT_MIB", 0)
+    assert flash.ds_heads_per_launch(lib, 1, 32, 1, 8192, 8192, 128) == 0
+
+
+def test_ds_workspace_allocation_failure_is_reported_as_none(monkeypatch):
+    from flagattention_amd import flash
+
+    def no_memory(*args, **kwargs):
+        raise torch.OutOfMemoryError("out of memory")
+
+    monkeypatch.setattr(flash.torch, "empty", no_memory)
+    assert flash._ds_workspace(_SizesOnly(), "cpu", 1, 32, 8192, 8192) is None
