@@ -11,8 +11,7 @@ import os
 import torch
 
 from . import _abi, _config, _lib
-from .split_kv import (num_splits_heuristic, split_kv_forward, SPLIT_BLOCK_M, SPLIT_BLOCK_N,
-                       DECODE_MAX_ROWS)
+from .split_kv import num_splits_heuristic, split_kv_forward, split_units, DECODE_MAX_ROWS
 from .total import _total_attention
 from .dropout import philox_cuda_seed_offset
 
@@ -89,7 +88,8 @@ class FlashAttention(torch.autograd.Function):
             else:
                 seed, offset = 0, 0
             dropout = (dropout_p, seed, offset)
-            splits = num_splits_heuristic(B, H, M, N, SPLIT_BLOCK_M, SPLIT_BLOCK_N, num_cus, 128)
+            split_block_m, split_block_n = split_units(B, H, M, N, D, causal)   # flash.py:59 of the reference
+            splits = num_splits_heuristic(B, H, M, N, split_block_m, split_block_n, num_cus, 128)
             if splits > 1:
                 assert not is_dropout, "Cannot apply dropout with splitkv."   # as flash.py:89
             if splits > 1 or (M <= DECODE_MAX_ROWS and N >= 1024 and not is_dropout):

@@ -9,11 +9,12 @@ import math
 
 import torch
 
-from . import _abi, _lib
+from . import _abi, _config, _lib
 
 __all__ = ["attention"]
 
 SPLIT_BLOCK_M, SPLIT_BLOCK_N = 16, 128
+FWD_TILES = ((SPLIT_BLOCK_M, SPLIT_BLOCK_N),)
 # Up to this many query positions the decode-shaped kernel is used even where the reference's rule
 # would not split: it multiplies 16-row tiles and reads K/V once per kv head, where the dense
 # forward kernel would fill 128-row tiles per query head with a handful of rows.
@@ -21,8 +22,15 @@ DECODE_MAX_ROWS = 16
 
 
 def get_fwd_config(B, H, M, N, D, causal):
-    """Informational (``split_kv.py:229-231`` hook): (BLOCK_M, BLOCK_N, num_stages, num_warps)."""
+    """(BLOCK_M, BLOCK_N, num_stages, num_warps): the overridable hook of ``split_kv.py:229-231``, called
+    before the split rule is evaluated (``split_kv.py:288``, ``flash.py:59``).  The split kernel is
+    compiled for one tile; any other answer is reported once and the compiled one is used."""
     return (SPLIT_BLOCK_M, SPLIT_BLOCK_N, 1, 4)
+
+
+def split_units(B, H, M, N, D, causal):
+    """(BLOCK_M, BLOCK_N) in which the split rule counts work: what the hook names, if compiled."""
+    return _config.resolve(get_fwd_config, FWD_TILES, "flash_attention split-kv forward", (B, H, M, N, D, causal))
 
 
 def num_splits_heuristic(B, H, M, N, block_m, block_n, num_cus, max_splits):
@@ -121,6 +129,7 @@ def attention(q, k, v, causal=False, sm_scale=None):
     lib = _lib.get()
     q, k, v = _abi.kernel_ready(q), _abi.kernel_ready(k), _abi.kernel_ready(v)
     with torch.cuda.device(q.device):
-        splits = num_splits_heuristic(B, H, M, N, SPLIT_BLOCK_M, SPLIT_BLOCK_N, lib.fa_num_cus(), 128)
+        block_m, block_n = split_units(B, H, M, N, D, causal)
+        splits = num_splits_heuristic(B, H, M, N, block_m, block_n, lib.fa_num_cus(), 128)
         o, _ = split_kv_forward(lib, q, k, v, causal, sm_scale, splits, single_direct=True)
     return o

@@ -6,17 +6,23 @@ import math
 
 import torch
 
-from . import _abi, _lib
+from . import _abi, _config, _lib
+
+# (BLOCK_M, BLOCK_N) the kernel is compiled for: queries per pipeline step, keys per workgroup
+FWD_TILES = ((64, 128),)
 
 
 def get_fwd_config(B, H, M, N, D, causal):
-    """Informational (``total.py:6-7`` hook)."""
+    """(BLOCK_M, BLOCK_N, num_stages, num_warps): the overridable hook of ``total.py:6-7``, called before
+    every launch (``total.py:29``).  The kernel is compiled for one tile; any other answer is reported
+    once and the compiled one is launched."""
     return (64, 128, 2, 4)
 
 
 def _total_attention(lib, q, k, l, causal, sm_scale):
     B, H, M, D = q.shape
     N = k.shape[2]
+    _config.resolve(get_fwd_config, FWD_TILES, "total_attention", (B, H, M, N, D, causal))
     tot = torch.empty((B, H, N), dtype=torch.float32, device=q.device)
     _abi.fa_total_attn(lib, q, k, l, tot, causal, sm_scale)
     return tot

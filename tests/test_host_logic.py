@@ -185,3 +185,27 @@ def test_ds_workspace_allocation_failure_is_reported_as_none(monkeypatch):
 
     monkeypatch.setattr(flash.torch, "empty", no_memory)
     assert flash._ds_workspace(_SizesOnly(), "cpu", 1, 32, 8192, 8192) is None
+
+
+def test_split_and_total_hooks_are_live(monkeypatch):
+    """Replacing ``split_kv.get_fwd_config`` / ``total.get_fwd_config`` takes effect at the next call
+    (the reference reads them at ``split_kv.py:288``, ``flash.py:59`` and ``total.py:29``)."""
+    import warnings
+    from flagattention_amd import _config, split_kv, total
+    assert split_kv.split_units(1, 8, 1, 4096, 128, False) == (16, 128)
+    calls = []
+
+    def mine(B, H, M, N, D, causal):
+        calls.append((B, H, M, N, D, causal))
+        return (32, 64, 2, 8)
+
+    monkeypatch.setattr(split_kv, "get_fwd_config", mine)
+    monkeypatch.setattr(_config, "_warned", set())
+    with warnings.catch_warnings(record=True) as caught:
+        warnings.simplefilter("always")
+        assert split_kv.split_units(1, 8, 1, 4096, 128, False) == (16, 128)   # not compiled: said once, default used
+        assert split_kv.split_units(1, 8, 1, 4096, 128, False) == (16, 128)
+    assert calls == [(1, 8, 1, 4096, 128, False)] * 2
+    assert len([w for w in caught if "BLOCK_M=32" in str(w.message)]) == 1
+    # the default hooks name the compiled tiles
+    assert tuple(total.get_fwd_config(1, 8, 128, 128, 64, True)[:2]) in total.FWD_TILES

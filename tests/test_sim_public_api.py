@@ -1,0 +1,165 @@
+"""The public operators (``flag_attn.flash_attention`` / ``piecewise_attention`` / ``paged_attention``)
+end to end on the host lane simulator: the same Python host logic the GPU path runs -- hooks, split
+decision, dS hand-over policy, slicing, autograd wiring, group sums -- with CPU tensors and the kernel
+sources compiled for the simulator.  Two test-only substitutions make that possible: the library
+handle is the simulator build, and ``torch.cuda.device`` (a no-op for these tensors) is a null context.
+The shipped package has no such path: without the HIP library it raises.
+"""
+import contextlib
+import math
+
+import pytest
+import torch
+
+import flag_attn
+from flagattention_amd import _lib, flash, piecewise
+from oracle import flash_attention as oracle_flash, paged_attention as oracle_paged, piecewise_attention as oracle_pw
+from oracle import within_two_x
+from tests.sim import simlib
+
+torch.manual_seed(20240)
+
+
+@pytest.fixture(autouse=True)
+def simulator_behind_the_public_api(monkeypatch):
+    lib = simlib.get()
+    monkeypatch.setattr(_lib, "get", lambda: lib)
+    monkeypatch.setattr(torch.cuda, "device", lambda device: contextlib.nullcontext())
+    return lib
+
+
+def check(name, hyp, same, ref, strict=False):
+    ok, e_hyp, e_same = within_two_x(hyp, same, ref, strict=strict)
+    assert ok, f"{name}: kernel err {e_hyp:.3e} vs same-precision torch err {e_same:.3e}"
+
+
+def rnd(*shape, dtype=torch.bfloat16, grad=False):
+    t = torch.randn(*shape).to(dtype)
+    return t.requires_grad_() if grad else t
+
+
+def flash_case(B, H, Hk, M, N, D, causal, dtype=torch.bfloat16):
+    q, k, v = rnd(B, H, M, D, dtype=dtype, grad=True), rnd(B, Hk, N, D, dtype=dtype, grad=True), rnd(B, Hk, N, D, dtype=dtype, grad=True)
+    do = rnd(B, H, M, D, dtype=dtype)
+    ref = oracle_flash(q, k, v, causal, upcast=True, return_log_normalizer=True, return_total_attention=True)
+    same = oracle_flash(q, k, v, causal, upcast=False, return_log_normalizer=True, return_total_attention=True)
+    g_ref = torch.autograd.grad(ref[0], (q, k, v), do)
+    g_same = torch.autograd.grad(same[0], (q, k, v), do)
+    return (q, k, v, do), ref, same, g_ref, g_same
+
+
+@pytest.mark.parametrize("B,H,Hk,M,N,D,causal", [
+    (1, 4, 2, 70, 90, 64, True),       # grouped heads: dK/dV summed over each kv head's query heads
+    (2, 2, 2, 65, 40, 128, False),
+    (1, 2, 1, 40, 130, 32, True),
+])
+def test_flash_attention_forward_backward(B, H, Hk, M, N, D, causal):
+    (q, k, v, do), ref, same, g_ref, g_same = flash_case(B, H, Hk, M, N, D, causal)
+    o, L, tot, seed, offset = flag_attn.flash_attention(q, k, v, causal=causal, return_log_normalizer=True,
+                                                        return_total_attention=True)
+    assert seed is None and offset is None
+    grads = torch.autograd.grad(o, (q, k, v), do)
+    check("o", o, same[0], ref[0], strict=True)
+    check("L", L, same[1], ref[1])
+    check("total", tot, same[2], ref[2])
+    for name, h, s, r in zip(("dq", "dk", "dv"), grads, g_same, g_ref):
+        assert h.shape == r.shape and h.dtype == s.dtype
+        check(name, h, s, r, strict=True)
+    # plain call: the tensor alone (flash.py:150-160 of the reference)
+    assert torch.equal(flag_attn.flash_attention(q, k, v, causal=causal), o)
+
+
+@pytest.mark.parametrize("route", ["whole", "sliced", "recompute", "no memory"])
+def test_flash_backward_routes_agree(monkeypatch, route):
+    """The dS hand-over, its sliced form, the recomputing pair and the fall-back taken when the workspace
+    cannot be allocated are four ways through ``FlashAttention.backward``; all meet the 2x rule and the
+    two hand-over forms agree bit for bit."""
+    B, H, Hk, M, N, D = 2, 4, 2, 64, 96, 128
+    (q, k, v, do), ref, same, g_ref, g_same = flash_case(B, H, Hk, M, N, D, True)
+    heads = {"whole": B * H, "sliced": 2, "recompute": 0, "no memory": B * H}[route]
+    monkeypatch.setattr(flash, "ds_heads_per_launch", lambda *a, **kw: heads)
+    if route == "no memory":
+        monkeypatch.setattr(flash, "_ds_workspace", lambda *a, **kw: None)
+    o = flag_attn.flash_attention(q, k, v, causal=True)
+    grads = torch.autograd.grad(o, (q, k, v), do)
+    for name, h, s, r in zip(("dq", "dk", "dv"), grads, g_same, g_ref):
+        check(name, h, s, r, strict=True)
+    if route == "sliced":
+        monkeypatch.setattr(flash, "ds_heads_per_launch", lambda *a, **kw: B * H)
+        whole = torch.autograd.grad(flag_attn.flash_attention(q, k, v, causal=True), (q, k, v), do)
+        for a, b in zip(grads, whole):
+            assert torch.equal(a, b)
+
+
+def test_flash_attention_decode_shape_takes_the_split_path(monkeypatch):
+    calls = []
+    real = flash.split_kv_forward
+    monkeypatch.setattr(flash, "split_kv_forward", lambda *a, **kw: (calls.append(1), real(*a, **kw))[1])
+    q, k, v = rnd(1, 4, 1, 64, dtype=torch.float16), rnd(1, 2, 1100, 64, dtype=torch.float16), rnd(1, 2, 1100, 64, dtype=torch.float16)
+    o, L, *_ = flag_attn.flash_attention(q, k, v, causal=False, return_log_normalizer=True)
+    assert calls
+    ref = oracle_flash(q, k, v, False, upcast=True, return_log_normalizer=True)
+    same = oracle_flash(q, k, v, False, upcast=False, return_log_normalizer=True)
+    check("o", o, same[0], ref[0])
+    check("L", L, same[1], ref[1])
+    # the forward-only entry point of split_kv.py:266-330
+    o2 = flag_attn.flash_attention_split_kv(q, k, v, causal=False)
+    check("o (split_kv entry)", o2, same[0], ref[0])
+
+
+def test_replaced_hooks_are_called_per_launch(monkeypatch):
+    seen = []
+
+    def fwd(B, H, M, N, D, causal):
+        seen.append(("fwd", B, H, M, N, D, causal))
+        return (128, 64, 2, 4)
+
+    def bwd(B, H, M, N, D, causal):
+        seen.append(("bwd", B, H, M, N, D, causal))
+        return (64, 128, 3, 4)
+
+    monkeypatch.setattr(flash, "get_fwd_config", fwd)
+    monkeypatch.setattr(flash, "get_bwd_config", bwd)
+    q, k, v = rnd(1, 2, 40, 32, grad=True), rnd(1, 2, 50, 32, grad=True), rnd(1, 2, 50, 32, grad=True)
+    o = flag_attn.flash_attention(q, k, v, causal=True)
+    torch.autograd.grad(o, (q, k, v), torch.ones_like(o))
+    assert seen == [("fwd", 1, 2, 40, 50, 32, True), ("bwd", 1, 2, 40, 50, 32, True)]
+
+
+@pytest.mark.parametrize("route", ["whole", "sliced", "recompute", "no memory"])
+def test_piecewise_attention_routes(monkeypatch, route):
+    B, H, M, N, D, w = 1, 2, 70, 70, 128, 24
+    ins = [rnd(B, H, M if i in (0, 2) else N, D, grad=True) for i in range(5)]   # q1, k1, q2, k2, v
+    do = rnd(B, H, M, D)
+    heads = {"whole": B * H, "sliced": 1, "recompute": 0, "no memory": B * H}[route]
+    monkeypatch.setattr(piecewise, "ds_heads_per_launch", lambda *a, **kw: heads)
+    if route == "no memory":
+        monkeypatch.setattr(piecewise, "_ds_workspace", lambda *a, **kw: None)
+    o = flag_attn.piecewise_attention(*ins, w, causal=True)
+    grads = torch.autograd.grad(o, ins, do)
+    ref = oracle_pw(*ins, w, causal=True, upcast=True)
+    same = oracle_pw(*ins, w, causal=True)
+    g_ref = torch.autograd.grad(ref, ins, do)
+    g_same = torch.autograd.grad(same, ins, do)
+    check("o", o, same, ref)
+    for name, h, s, r in zip(("dq1", "dk1", "dq2", "dk2", "dv"), grads, g_same, g_ref):
+        check(name, h, s, r)
+
+
+def test_paged_attention_public_call():
+    seqs, Hq, Hkv, D, bs = 3, 4, 2, 64, 16
+    ctx = torch.tensor([37, 1, 160], dtype=torch.int32)
+    blocks = [(int(c) + bs - 1) // bs for c in ctx]
+    num_blocks = sum(blocks) + 2
+    perm = torch.randperm(num_blocks)
+    table = torch.zeros(seqs, max(blocks), dtype=torch.int32)
+    at = 0
+    for s, n in enumerate(blocks):
+        table[s, :n] = perm[at:at + n]
+        at += n
+    q = rnd(seqs, Hq, D, dtype=torch.float16)
+    kc, vc = rnd(num_blocks, Hkv, bs, D, dtype=torch.float16), rnd(num_blocks, Hkv, bs, D, dtype=torch.float16)
+    scale = D ** -0.5
+    out = flag_attn.paged_attention(q, kc, vc, ctx, table, scale, int(ctx.max()))
+    ref = oracle_paged(q.float(), kc.float(), vc.float(), table, ctx, scale)
+    assert torch.allclose(out.float(), ref, atol=2e-3, rtol=1e-5)   # tests/flag_attn/test_paged_attention.py:62
