@@ -5,12 +5,12 @@
 // launches whose tile config is BLOCK_M = 256 (flash.py:64-87); fa_fwd.hip holds the 128-row kernel.
 //
 // Why a second forward kernel.  With 32 query rows per wavefront every matrix instruction needs a
-// fresh 1 KB operand from LDS, which at full matrix rate is exactly the LDS bandwidth of a compute
-// unit: the 128-row kernel is bound by LDS.  Here a wavefront owns two 32-row blocks (A and B), so one
-// K (or V^T) operand read from LDS feeds two matrix instructions.  That takes most of the register
-// file (O^T: 128, Q: 64, S: 64, P: 32), i.e. ONE wavefront per SIMD, so nothing but the wavefront
-// itself can fill the matrix pipe while it does the softmax.  The overlap therefore comes from the
-// instruction order, which is fixed by hand:
+// fresh 1 KB operand from LDS (1.8 LDS instructions per matrix instruction, counting the transposing
+// reads).  Here a wavefront owns two 32-row blocks (A and B), so one K (or V^T) operand read from LDS
+// feeds two matrix instructions (0.75 per matrix instruction; the cycles spent waiting for LDS fall
+// to a sixth).  That takes most of the register file (O^T: 128, Q: 64, S: 64, P: 32), i.e. ONE
+// wavefront per SIMD, so nothing but the wavefront itself can fill the matrix pipe while it does the
+// softmax.  The overlap therefore comes from the instruction order, which is fixed by hand:
 //
 //   * An iteration i issues 64 matrix instructions in four runs of 16:
 //         S(i+1) keys 0-31 | O += V(i)^T P(i) keys 0-31 | S(i+1) keys 32-63 | O += V(i)^T P(i) keys 32-63
