@@ -117,6 +117,10 @@ FA_DEVICE void decode_block(const Src& src, const T* q_row /* query row of lane 
   // Branch-free on purpose: a guarded load would put every chunk in its own basic block, and the
   // compiler then waits for ALL outstanding loads before each one.  Rows past the end are read from
   // the last valid row instead; their scores are masked, and finite values times zero stay zero.
+  // Precondition that follows: the value rows of every key in [n_begin, n_end) are finite, including
+  // keys that only the causal limit hides from some query row -- they enter the second product with
+  // probability 0.  The reference's kernels form the same product p @ v with p = 0 at those
+  // positions (flash.py:448-461, split_kv.py:137), so a non-finite value there gives NaN in both.
   static_assert(C::TK * C::CPR == 64 * C::CH, "a step is a whole number of 64-lane load instructions");
   auto fetch = [&](int n0, u32x4* kst, u32x4* vst) {
 #pragma unroll
