@@ -35,7 +35,9 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E peak
 # HBM traffic per launch at the default workloads, from rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE,
 # KiB per dispatch), each scaled by what the same counter reads for a plain 1 GiB device copy
 # (FETCH_SIZE reads 0.5 GiB for 1 GiB fetched -> x2.0; WRITE_SIZE reads 1.0 GiB -> x1.0);
-# profiles/hbm_traffic_dkdv_and_paged_pmc.txt.
+# profiles/hbm_traffic_dkdv_and_paged_pmc.txt.  The dK/dV and paged kernels move the same bytes as when
+# these were taken (their later changes reorder instructions and the scan of the context lengths); the
+# legs without such a measurement report traffic = null.
 DKDV_TRAFFIC_BYTES = int((2.0 * 3.631e5 + 1.0 * 1.311e5) * 1024)      # recomputing path: 744 MB read + 134 MB written
 DKDV_DS_TRAFFIC_BYTES = int((2.0 * 3.604e5 + 1.0 * 2.236e6) * 1024)   # dS kept: 738 MB read + 2.29 GB written
 PAGED_TRAFFIC_BYTES = int((2.0 * 5.014e5 + 1.0 * 4010) * 1024)        # 1.027 GB read + 4 MB written
