@@ -40,7 +40,6 @@ FA_DEVICE int thread_id() { return (int)threadIdx.x; }
 FA_DEVICE int block_x() { return (int)blockIdx.x; }
 FA_DEVICE int block_y() { return (int)blockIdx.y; }
 FA_DEVICE int block_z() { return (int)blockIdx.z; }
-FA_DEVICE int grid_x() { return (int)gridDim.x; }
 FA_DEVICE int grid_z() { return (int)gridDim.z; }
 FA_DEVICE void block_sync() { __syncthreads(); }
 // The workgroup barrier alone, without the memory fence of block_sync(): for code that has already
@@ -77,88 +76,6 @@ FA_DEVICE f32x16 mfma32_vacc(bf16x8 a, bf16x8 b, f32x16 c) {
   asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "a"(b));
   return c;
 }
-// First product of a chain with the accumulator pinned to VGPRs: D = A * B (no accumulator to read).
-FA_DEVICE f32x16 mfma32_vacc_first(half8 a, half8 b) {
-  f32x16 c;
-  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "a"(b));
-  return c;
-}
-FA_DEVICE f32x16 mfma32_vacc_first(bf16x8 a, bf16x8 b) {
-  f32x16 c;
-  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "a"(b));
-  return c;
-}
-// The product with the accumulator pinned to AGPRs and both operands in VGPRs (an output accumulator
-// that the vector ALU touches only in rare rescales and at the end).  As with mfma32_vacc the compiler
-// does not know that this is a matrix instruction: a CALLER that reads the accumulator with ordinary
-// code afterwards first lets the pipe drain (mfma_drain()).
-FA_DEVICE void mfma32_aacc(half8 a, half8 b, f32x16& c) {
-  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
-}
-FA_DEVICE void mfma32_aacc(bf16x8 a, bf16x8 b, f32x16& c) {
-  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
-}
-// Chain instructions with accumulator and both operands in VGPRs.
-FA_DEVICE f32x16 mfma32_vvv_first(half8 a, half8 b) {
-  f32x16 c;
-  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
-  return c;
-}
-FA_DEVICE f32x16 mfma32_vvv_first(bf16x8 a, bf16x8 b) {
-  f32x16 c;
-  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
-  return c;
-}
-FA_DEVICE f32x16 mfma32_vvv(half8 a, half8 b, f32x16 c) {
-  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
-  return c;
-}
-FA_DEVICE f32x16 mfma32_vvv(bf16x8 a, bf16x8 b, f32x16 c) {
-  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
-  return c;
-}
-// Chain instructions with both operands in AGPRs (LDS reads can target AGPRs directly; a register-resident
-// operand is moved there once) and the accumulator in VGPRs.
-// (the first product of a chain names its accumulator as read-write although it only writes it: the
-// accumulator then stays one long-lived value in one place for the register allocator)
-FA_DEVICE void mfma32_vaa_first(half8 a, half8 b, f32x16& c) {
-  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "+v"(c) : "a"(a), "a"(b));
-}
-FA_DEVICE void mfma32_vaa_first(bf16x8 a, bf16x8 b, f32x16& c) {
-  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "+v"(c) : "a"(a), "a"(b));
-}
-FA_DEVICE void mfma32_vaa(half8 a, half8 b, f32x16& c) {
-  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "a"(a), "a"(b));
-}
-FA_DEVICE void mfma32_vaa(bf16x8 a, bf16x8 b, f32x16& c) {
-  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "a"(a), "a"(b));
-}
-// Accumulator and A operand in AGPRs, B operand in VGPRs.
-FA_DEVICE void mfma32_aav(half8 a, half8 b, f32x16& c) {
-  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "a"(a), "v"(b));
-}
-FA_DEVICE void mfma32_aav(bf16x8 a, bf16x8 b, f32x16& c) {
-  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "a"(a), "v"(b));
-}
-// The same two chain instructions with the accumulator in AGPRs (B operand in AGPRs as well).
-FA_DEVICE f32x16 mfma32_aacc_first(half8 a, half8 b) {
-  f32x16 c;
-  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&a"(c) : "v"(a), "a"(b));
-  return c;
-}
-FA_DEVICE f32x16 mfma32_aacc_first(bf16x8 a, bf16x8 b) {
-  f32x16 c;
-  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&a"(c) : "v"(a), "a"(b));
-  return c;
-}
-FA_DEVICE f32x16 mfma32_aacc_ab(half8 a, half8 b, f32x16 c) {
-  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "a"(b));
-  return c;
-}
-FA_DEVICE f32x16 mfma32_aacc_ab(bf16x8 a, bf16x8 b, f32x16 c) {
-  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "a"(b));
-  return c;
-}
 // max(a, b, c) and max(a, b) as single instructions (no canonicalisation of the inputs: callers pass
 // matrix-instruction results and values derived from them)
 FA_DEVICE float max3(float a, float b, float c) {
@@ -170,22 +87,6 @@ FA_DEVICE float max2(float a, float b) {
   float r;
   asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
   return r;
-}
-// Element access to an accumulator that lives in AGPRs, spelled out so that the compiler never sees a
-// vector-ALU use of it (which would make it keep the accumulator in VGPRs and copy it around every
-// matrix instruction).
-template <int R> FA_DEVICE float acc_read(const f32x16& c) {
-  float x;
-  asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(x) : "a"(c[R]));
-  return x;
-}
-template <int R> FA_DEVICE void acc_scale(f32x16& c, float f) {
-  float t;
-  asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 1\n\tv_accvgpr_write_b32 %0, %1"
-               : "+a"(c[R]), "=&v"(t) : "v"(f));
-}
-template <int R> FA_DEVICE void acc_clear(f32x16& c) {
-  asm volatile("v_accvgpr_write_b32 %0, 0" : "=a"(c[R]));
 }
 // More wait states than any matrix instruction needs before its result may be read by other units.
 FA_DEVICE void mfma_drain() { asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 7" ::: "memory"); }
@@ -310,16 +211,6 @@ FA_DEVICE uint32_t pack2(bf16_t, float a, float b) {
   typedef __bf16 b2 __attribute__((ext_vector_type(2)));
   b2 v; v[0] = (__bf16)a; v[1] = (__bf16)b;
   return __builtin_bit_cast(uint32_t, v);
-}
-FA_DEVICE float add_pair(half_t, uint32_t pair, float acc) {
-  typedef _Float16 h2 __attribute__((ext_vector_type(2)));
-  h2 one; one[0] = (_Float16)1.f; one[1] = (_Float16)1.f;
-  return __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, pair), one, acc, false);
-}
-FA_DEVICE float add_pair(bf16_t, uint32_t pair, float acc) {
-  typedef __bf16 b2 __attribute__((ext_vector_type(2)));
-  b2 one; one[0] = (__bf16)1.f; one[1] = (__bf16)1.f;
-  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(b2, pair), one, acc, false);
 }
 
 }  // namespace hw

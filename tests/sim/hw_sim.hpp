@@ -212,7 +212,6 @@ inline int thread_id() { return hwsim::cur; }
 inline int block_x() { return hwsim::bx; }
 inline int block_y() { return hwsim::by; }
 inline int block_z() { return hwsim::bz; }
-inline int grid_x() { return hwsim::gx; }
 inline void store_streaming(void* p, u32x4 v) { *(u32x4*)p = v; }
 inline u32x4 load_streaming(const void* p) { return *(const u32x4*)p; }
 inline void wait_global_loads() {}
@@ -235,24 +234,6 @@ template <class V8> inline f32x16 mfma32_any(V8 a, V8 b, f32x16 c) {
 inline f32x16 mfma32(half8 a, half8 b, f32x16 c) { return mfma32_any(a, b, c); }
 inline f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) { return mfma32_any(a, b, c); }
 inline f32x16 zero16() { f32x16 z; for (int r = 0; r < 16; ++r) z[r] = 0.f; return z; }
-inline f32x16 mfma32_vacc_first(half8 a, half8 b) { return mfma32_any(a, b, zero16()); }
-inline f32x16 mfma32_vacc_first(bf16x8 a, bf16x8 b) { return mfma32_any(a, b, zero16()); }
-inline void mfma32_aacc(half8 a, half8 b, f32x16& c) { c = mfma32_any(a, b, c); }
-inline void mfma32_aacc(bf16x8 a, bf16x8 b, f32x16& c) { c = mfma32_any(a, b, c); }
-inline f32x16 mfma32_aacc_first(half8 a, half8 b) { return mfma32_any(a, b, zero16()); }
-inline f32x16 mfma32_aacc_first(bf16x8 a, bf16x8 b) { return mfma32_any(a, b, zero16()); }
-inline f32x16 mfma32_aacc_ab(half8 a, half8 b, f32x16 c) { return mfma32_any(a, b, c); }
-inline f32x16 mfma32_aacc_ab(bf16x8 a, bf16x8 b, f32x16 c) { return mfma32_any(a, b, c); }
-inline f32x16 mfma32_vvv_first(half8 a, half8 b) { return mfma32_any(a, b, zero16()); }
-inline f32x16 mfma32_vvv_first(bf16x8 a, bf16x8 b) { return mfma32_any(a, b, zero16()); }
-inline f32x16 mfma32_vvv(half8 a, half8 b, f32x16 c) { return mfma32_any(a, b, c); }
-inline f32x16 mfma32_vvv(bf16x8 a, bf16x8 b, f32x16 c) { return mfma32_any(a, b, c); }
-inline void mfma32_vaa_first(half8 a, half8 b, f32x16& c) { c = mfma32_any(a, b, zero16()); }
-inline void mfma32_vaa_first(bf16x8 a, bf16x8 b, f32x16& c) { c = mfma32_any(a, b, zero16()); }
-inline void mfma32_vaa(half8 a, half8 b, f32x16& c) { c = mfma32_any(a, b, c); }
-inline void mfma32_vaa(bf16x8 a, bf16x8 b, f32x16& c) { c = mfma32_any(a, b, c); }
-inline void mfma32_aav(half8 a, half8 b, f32x16& c) { c = mfma32_any(a, b, c); }
-inline void mfma32_aav(bf16x8 a, bf16x8 b, f32x16& c) { c = mfma32_any(a, b, c); }
 // accumulator tuples that the GPU build pins to fixed physical registers: plain values here
 template <int I, class V8> inline void pinned_o_mfma(V8 a, V8 b, f32x16& c) { c = mfma32_any(a, b, c); }
 template <int I, class V8> inline void pinned_s_mfma_first(V8 a, V8 b, f32x16& c) { c = mfma32_any(a, b, zero16()); }
@@ -261,9 +242,6 @@ template <int I> inline void pinned_o_clear(f32x16& c) { c = zero16(); }
 template <int I> inline void pinned_o_scale(f32x16& c, float f) { for (int r = 0; r < 16; ++r) c[r] *= f; }
 template <int I, int R> inline float pinned_o_read(const f32x16& c) { return c[R]; }
 inline void mfma_drain() {}
-template <int R> inline float acc_read(const f32x16& c) { return c[R]; }
-template <int R> inline void acc_scale(f32x16& c, float f) { c[R] *= f; }
-template <int R> inline void acc_clear(f32x16& c) { c[R] = 0.f; }
 inline f32x16 mfma32_vacc(half8 a, half8 b, f32x16 c) { return mfma32_any(a, b, c); }
 inline f32x16 mfma32_vacc(bf16x8 a, bf16x8 b, f32x16 c) { return mfma32_any(a, b, c); }
 
@@ -353,12 +331,6 @@ inline uint32_t pack2(half_t, float a, float b) {
 inline uint32_t pack2(bf16_t, float a, float b) {
   bf16_t v[2] = {(bf16_t)a, (bf16_t)b};
   uint32_t r; memcpy(&r, v, 4); return r;
-}
-inline float add_pair(half_t, uint32_t pair, float acc) {
-  half_t v[2]; memcpy(v, &pair, 4); return acc + (float)v[0] + (float)v[1];
-}
-inline float add_pair(bf16_t, uint32_t pair, float acc) {
-  bf16_t v[2]; memcpy(v, &pair, 4); return acc + (float)v[0] + (float)v[1];
 }
 inline bool wave_any(bool pred) {
   float v = pred ? 1.f : 0.f;
