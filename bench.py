@@ -14,9 +14,15 @@ The JSON line also carries
     MFMA peak, its launches timed with HIP events on the stream they run on;
   * ``cpu_baseline``: the plain-torch fp32 oracle timed on the host cores on a bounded sample
     (a few heads of the same workload);
-  * ``kernels``: every launch of a step with its own counted FLOPs and time;
+  * ``kernels``: every launch of a step with its own counted FLOPs and time (median over 5 groups of
+    20 back-to-back launches, HIP events on the launch stream);
+  * ``other_flash_workloads``: the remaining flash configurations of the workload list as records of
+    their own (B=4 H=16 T=2048; head size 64; Tq=1024 against Tk=8192), forward + backward through
+    the public API;
   * ``paged_decode``: the paged-attention decode configuration (64 sequences, 32 query / 8 kv heads,
-    head 128, block 16, context lengths uniform in [512, 8192]) as achieved HBM GB/s.
+    head 128, block 16, context lengths uniform in [512, 8192]) as achieved HBM GB/s;
+  * ``splitkv_decode`` (dense decode over 32768 keys, three K/V sets in rotation so that no launch is
+    served from the last-level cache), ``piecewise`` and ``total_attention`` with rooflines of their own.
 """
 import argparse
 import json
