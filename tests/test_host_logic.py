@@ -209,3 +209,20 @@ def test_split_and_total_hooks_are_live(monkeypatch):
     assert len([w for w in caught if "BLOCK_M=32" in str(w.message)]) == 1
     # the default hooks name the compiled tiles
     assert tuple(total.get_fwd_config(1, 8, 128, 128, 64, True)[:2]) in total.FWD_TILES
+
+
+def test_bench_counts_the_flops_of_the_quoted_workloads():
+    """bench.py's FLOP counts against the figures of the workload list: forward 2 products, backward 5,
+    each 2 * B * H * pairs * D with `pairs` the unmasked (query, key) pairs of the bottom-right aligned mask."""
+    import bench
+    assert bench.causal_pairs(8192, 8192) == 8192 * 8193 // 2
+    assert bench.causal_pairs(4, 6) == 3 + 4 + 5 + 6            # every query sees the 2 extra keys
+    assert bench.causal_pairs(6, 4) == 0 + 0 + 1 + 2 + 3 + 4    # the first rows see nothing
+    assert bench.causal_pairs(1024, 8192) == 1024 * 7168 + 1024 * 1025 // 2
+    c3 = bench.WORKLOADS["c3"]
+    x = 2.0 * c3["B"] * c3["H"] * bench.causal_pairs(c3["T"], c3["T"]) * c3["D"]
+    assert abs(7 * x / 1e9 - 1924.4) < 0.3          # 549.8 forward + 1374.5 backward
+    c2 = bench.WORKLOADS["c2"]
+    x2 = 2.0 * c2["B"] * c2["H"] * bench.causal_pairs(c2["T"], c2["T"]) * c2["D"]
+    assert abs(7 * x2 / 1e9 - 240.6) < 0.2
+    assert bench.PEAK_BF16_TFLOPS == 2500.0 and bench.PEAK_HBM_GBS == 8000.0
