@@ -60,7 +60,8 @@ struct WideCfg {
 // product of a half's S run sits in slot 15 (+ 32); a slot issues its matrix instruction first and its
 // vector work after it, so vector work in slot 17 follows two further matrix instructions, the first of
 // which cannot issue before the S product has left the front of the pipe and the second not before it
-// has written back.
+// has written back.  (Iteration -1 has no matrix instructions behind its S run and waits explicitly
+// there; tests/test_emitted_hazard_distances.py checks the distances in the emitted code.)
 static_assert(WideCfg::kMax >= 15 + 2, "the row maximum reads S before its last product has written back");
 static_assert(WideCfg::kMax + 8 <= WideCfg::kSwap && WideCfg::kSwap + 3 <= WideCfg::kFinal &&
               WideCfg::kFinal + 2 <= WideCfg::kExp0, "maximum, exchange, decision and first exponential in this order");
@@ -234,6 +235,9 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, 1) fa_fwd_wide_kernel(FwdParams p) {
           hw::pinned_o_mfma<4 * x + db>(ring[q % 4], hw::as_v8<T>(P[x][g]), O[x][db]);
         }
       }
+      // Iteration -1 has no second product: the slots behind its S run hold no matrix instruction, and the
+      // vector work of slot kMax would follow the run's last products too closely (hazard distances above)
+      if constexpr (DO_S && !DO_PV && kl == 16) hw::mfma_drain();
       // ------------------------------------------------- operand of the slot pair kLead ahead
       if constexpr (k % 2 == 0) {
         constexpr int q = (k + C::kLead) / 2;
