@@ -5,8 +5,8 @@ no wait states between such an instruction and a vector-ALU read of its result; 
 distance (static_asserts over the slot constants in fa_bwd.hip and fa_fwd_wide.hip).  Those asserts speak
 about the source.  The compiler, however, moves side-effect-free vector work across the scheduling fences,
 so this test looks at the built objects: it disassembles the gfx950 code of the two kernels' object files
-and checks, for every instruction that reads a VGPR last written by a matrix instruction, that enough
-wait states lie in between.  An 8-pass matrix instruction (32x32x16) needs its 8 passes plus 3 before the
+and checks, for every instruction that reads a vector register (VGPR or AGPR) last written by a matrix
+instruction, that enough wait states lie in between.  An 8-pass matrix instruction (32x32x16) needs its 8 passes plus 3 before the
 vector ALU may read the result; an instruction counts as one wait state, `s_nop N` as N + 1, and a matrix
 instruction in between as 8 (it cannot issue before the pipe has taken the one before it).
 """
@@ -22,16 +22,17 @@ BUILD = os.path.join(ROOT, "flagattention_amd", "csrc", "build")
 LLVM = "/opt/rocm/llvm/bin"
 NEEDED_WAIT_STATES = 11
 
-_RANGE = re.compile(r"\bv\[(\d+):(\d+)\]")
-_SINGLE = re.compile(r"\bv(\d+)\b")
+_RANGE = re.compile(r"\b([va])\[(\d+):(\d+)\]")
+_SINGLE = re.compile(r"\b([va])(\d+)\b")
 
 
 def _vgprs(operand):
+    """Vector registers named by an operand, both files: ('v', n) and ('a', n)."""
     regs = set()
-    for lo, hi in _RANGE.findall(operand):
-        regs.update(range(int(lo), int(hi) + 1))
-    for r in _SINGLE.findall(_RANGE.sub("", operand)):
-        regs.add(int(r))
+    for file, lo, hi in _RANGE.findall(operand):
+        regs.update((file, n) for n in range(int(lo), int(hi) + 1))
+    for file, r in _SINGLE.findall(_RANGE.sub("", operand)):
+        regs.add((file, int(r)))
     return regs
 
 
@@ -56,7 +57,7 @@ def _disassemble(obj, tmp_path):
 def closest_read(instructions):
     """(wait states, reading instruction) of the read that follows the matrix instruction whose result it takes
     most closely; the body is walked twice so that reads at the top of a loop meet writes at its bottom."""
-    written = {}      # vgpr -> (wait-state clock, matrix-instruction count) at its last write by a matrix instruction
+    written = {}      # register -> (wait-state clock, matrix-instruction count) at its last write by a matrix instruction
     clock = matrix = 0
     worst = (10 ** 9, None)
     checked = 0
@@ -72,9 +73,8 @@ def closest_read(instructions):
             clock += 1
             if op.startswith("v_mfma"):
                 matrix += 1
-                if operands[0].strip().startswith("v"):
-                    for r in _vgprs(operands[0]):
-                        written[r] = (clock, matrix)
+                for r in _vgprs(operands[0]):
+                    written[r] = (clock, matrix)
                 continue
             if not op.startswith(("v_", "ds_", "global_", "buffer_")):
                 continue
@@ -106,7 +106,7 @@ def test_the_audit_sees_a_read_that_comes_too_early():
     assert closest_read(own_accumulator)[1] == 0
 
 
-@pytest.mark.parametrize("obj", ["fa_fwd_wide.o", "fa_bwd.o"])
+@pytest.mark.parametrize("obj", ["fa_fwd_wide.o", "fa_bwd.o", "fa_fwd.o", "fa_splitkv.o", "fa_total.o"])
 def test_vector_reads_of_matrix_results_keep_their_distance(obj, tmp_path):
     path = os.path.join(BUILD, obj)
     if not os.path.exists(path) or not all(shutil.which(os.path.join(LLVM, t)) for t in
@@ -115,10 +115,10 @@ def test_vector_reads_of_matrix_results_keep_their_distance(obj, tmp_path):
     kernels = _disassemble(path, tmp_path)
     audited = reads = 0
     for name, instructions in kernels.items():
-        if not any(re.match(r"v_mfma\S* v\[", ins) for ins in instructions):
-            continue      # no matrix instruction with a VGPR accumulator
+        if not any(ins.startswith("v_mfma") for ins in instructions):
+            continue
         (states, ins), checked = closest_read(instructions)
         audited += 1
         reads += checked
         assert states >= NEEDED_WAIT_STATES, f"{name}: `{ins}` reads a matrix result after {states} wait states"
-    assert audited >= 2 and reads >= 1000, f"{obj}: {audited} kernels with VGPR accumulators, {reads} reads checked"
+    assert audited >= 2 and reads >= 100, f"{obj}: {audited} kernels with matrix instructions, {reads} reads checked"
