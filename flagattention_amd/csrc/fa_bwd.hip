@@ -364,8 +364,8 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
         constexpr int kP0 = C::KSTEPS + 1, kD0 = NA + 1, kP1 = NA + C::KSTEPS + 1, kD1 = 2 * NA + 1;
         // hw::mfma32_vacc hides its result registers from the compiler's hazard handling, so the slot
         // order itself has to keep a vector-ALU read of sx / dpx behind the matrix instruction that
-        // wrote them last.  A 32x32x16 product occupies the matrix pipe for 16 passes and its result
-        // may be read 18 cycles' worth of wait states after its last pass; a slot issues its matrix
+        // wrote them last.  A 32x32x16 product occupies the matrix pipe for 8 passes of 4 cycles and its
+        // result may be read 12 wait states (the passes plus 4) after its issue; a slot issues its matrix
         // instruction first and its element-wise work after it.  If the chain's last product sits in
         // slot w, the product of slot w + 1 cannot issue before w has left the pipe's front and the
         // product of slot w + 2 cannot issue before w has written back, so element-wise work of slot
