@@ -3,7 +3,8 @@
 // TEST INFRASTRUCTURE.  Each lane of a workgroup is a ucontext fiber; a wavefront's 64 fibers are
 // run in turn up to their next collective operation (matrix multiply, transposing LDS read, lane
 // exchange, workgroup barrier), the operation is evaluated for the whole wavefront with the operand
-// layouts measured on gfx950, and the fibers resume.  LDS is a heap block of exactly the requested
+// layouts measured on gfx950, and the fibers resume.  The order in which the wavefronts of a workgroup
+// advance between barriers is selectable (Schedule below), to expose a missing barrier.  LDS is a heap block of exactly the requested
 // size, so AddressSanitizer sees every out-of-range LDS or global access a kernel would make.
 #pragma once
 #include <stdint.h>
@@ -137,9 +138,35 @@ inline void eval_wave(int base, Op op) {
   }
 }
 
+// How the wavefronts of a workgroup interleave.  Correctly synchronised kernels give the same result
+// under every schedule; HWSIM_SCHEDULE picks one: "lockstep" (default: each wavefront in turn up to its
+// next collective operation), "ahead" / "ahead_descending" (each wavefront runs on alone until it waits
+// at a barrier or exits, lowest or highest index first: the largest skew barriers allow), "random"
+// (runs of random length in random order, seeded by HWSIM_SEED).
+enum ScheduleMode { kLockstep, kAheadAscending, kAheadDescending, kRandom };
+struct Schedule {
+  ScheduleMode mode = kLockstep;
+  uint64_t rng = 1;
+  uint64_t next() { rng ^= rng << 13; rng ^= rng >> 7; rng ^= rng << 17; return rng; }
+};
+inline Schedule schedule_from_env() {
+  Schedule s;
+  const char* m = getenv("HWSIM_SCHEDULE");
+  if (!m || !*m || !strcmp(m, "lockstep")) s.mode = kLockstep;
+  else if (!strcmp(m, "ahead")) s.mode = kAheadAscending;
+  else if (!strcmp(m, "ahead_descending")) s.mode = kAheadDescending;
+  else if (!strcmp(m, "random")) s.mode = kRandom;
+  else die("HWSIM_SCHEDULE must be lockstep, ahead, ahead_descending or random");
+  const char* seed = getenv("HWSIM_SEED");
+  s.rng = 0x9E3779B97F4A7C15ull ^ (seed ? strtoull(seed, nullptr, 10) : 0);
+  if (!s.rng) s.rng = 1;
+  return s;
+}
+
 // Runs `fn` once per lane of every workgroup of the grid, one workgroup at a time.
 inline void run_grid(dim3 grid, int threads, size_t lds_bytes, std::function<void()> fn) {
   if (threads % 64) die("workgroup size must be a multiple of the wavefront size");
+  Schedule sched = schedule_from_env();
   body = fn;
   gx = (int)grid.x;
   gz = (int)grid.z;
@@ -164,18 +191,22 @@ inline void run_grid(dim3 grid, int threads, size_t lds_bytes, std::function<voi
         }
         for (auto& s : state) s = 0;
         for (;;) {
-          int done = 0, waiting = 0;
-          for (int w = 0; w < waves; ++w) {
-            if (state[w] == 2) { ++done; continue; }
-            if (state[w] == 1) { ++waiting; continue; }
-            for (int l = 0; l < 64; ++l) resume(w * 64 + l);
-            Op op = lanes[w * 64].op;
-            for (int l = 1; l < 64; ++l)
-              if (lanes[w * 64 + l].op != op) die("lanes of one wavefront reached different collective operations");
-            if (op == OP_DONE) { state[w] = 2; ++done; }
-            else if (op == OP_BARRIER) { state[w] = 1; ++waiting; }
-            else eval_wave(w * 64, op);
+          // One pass over the wavefronts in the order and with the run lengths of the chosen schedule.
+          for (int i = 0; i < waves; ++i) {
+            int w = sched.mode == kAheadDescending ? waves - 1 - i : sched.mode == kRandom ? (int)(sched.next() % waves) : i;
+            long run = sched.mode == kLockstep ? 1 : sched.mode == kRandom ? 1 + (long)(sched.next() % 48) : (1L << 60);
+            while (run-- > 0 && state[w] == 0) {
+              for (int l = 0; l < 64; ++l) resume(w * 64 + l);
+              Op op = lanes[w * 64].op;
+              for (int l = 1; l < 64; ++l)
+                if (lanes[w * 64 + l].op != op) die("lanes of one wavefront reached different collective operations");
+              if (op == OP_DONE) state[w] = 2;
+              else if (op == OP_BARRIER) state[w] = 1;
+              else eval_wave(w * 64, op);
+            }
           }
+          int done = 0, waiting = 0;
+          for (int s : state) { done += s == 2; waiting += s == 1; }
           if (done == waves) break;
           if (done + waiting == waves) {
             if (done) die("workgroup barrier reached by some wavefronts after others exited");

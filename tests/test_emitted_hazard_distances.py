@@ -182,6 +182,58 @@ def closest_access(lines):
     return worst, checked[0]
 
 
+def dma_in_flight_at(lines, stops=("s_barrier", "s_endpgm")):
+    """The `stops` instructions that some path reaches while a global-to-LDS transfer may still be in flight.
+    Such a transfer is counted like any vector-memory load but writes LDS, which the compiler does not know:
+    the kernel itself waits for vmcnt(0) before the barrier behind which other wavefronts read the tile, and
+    before it ends (the transfer must not outlive the workgroup's LDS allocation)."""
+    blocks = _blocks(lines)
+    found = []
+    entry = [None] * len(blocks)
+    if blocks:
+        entry[0] = False
+    work = [0] if blocks else []
+    while work:
+        n = work.pop()
+        instructions, succ = blocks[n]
+        flying = entry[n]
+        for ins in instructions:
+            op = ins.split(" ")[0]
+            if op.startswith("global_load_lds"):
+                flying = True
+            elif op == "s_waitcnt" and "vmcnt(0)" in ins:
+                flying = False
+            elif op in stops and flying and ins not in found:
+                found.append(ins)
+        for s in succ:
+            if entry[s] is None or (flying and not entry[s]):
+                entry[s] = flying
+                work.append(s)
+    return found
+
+
+def test_the_transfer_audit_sees_a_missing_wait():
+    load = "global_load_lds_dwordx4 v1, s[2:3]"
+    assert dma_in_flight_at([load, "s_waitcnt vmcnt(0)", "s_barrier", "s_endpgm"]) == []
+    assert dma_in_flight_at([load, "s_waitcnt lgkmcnt(0)", "s_barrier", "s_waitcnt vmcnt(0)", "s_endpgm"]) == ["s_barrier"]
+    assert dma_in_flight_at([load, "s_waitcnt vmcnt(1)", "s_endpgm"]) == ["s_endpgm"]
+    loop = ["L0:", "s_barrier", load, "s_cbranch_scc1 L0", "s_waitcnt vmcnt(0)", "s_endpgm"]      # over the back edge
+    assert dma_in_flight_at(loop) == ["s_barrier"]
+
+
+def test_transfers_into_lds_have_landed_at_every_barrier_and_at_the_end(tmp_path):
+    path = os.path.join(BUILD, "fa_fwd_wide.o")
+    if not os.path.exists(path) or not all(shutil.which(os.path.join(LLVM, t)) for t in
+                                           ("llvm-objcopy", "clang-offload-bundler", "llvm-objdump")):
+        pytest.skip("needs the objects of a library build and the LLVM binary tools")
+    audited = 0
+    for name, lines in _disassemble(path, tmp_path).items():
+        if any(line.startswith("global_load_lds") for line in lines):
+            audited += 1
+            assert dma_in_flight_at(lines) == [], name
+    assert audited == 2       # the f16 and the bf16 kernel
+
+
 PRODUCT = "v_mfma_f32_32x32x16_bf16 v[192:207], v[2:5], a[0:3], v[192:207]"
 OTHER = "v_mfma_f32_32x32x16_bf16 a[0:15], v[2:5], v[6:9], a[0:15]"
 READ = "v_max_f32 v2, v192, v193"
