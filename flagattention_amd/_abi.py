@@ -31,14 +31,11 @@ def stream_of(t):
     return ctypes.c_void_p(0)
 
 
-def _stride(t, dim):
-    # the stride of a dimension of extent 1 is never used; torch leaves arbitrary values there
-    return t.stride(dim) if t.shape[dim] > 1 else 0
-
-
 def view4(t):
-    assert t.dim() == 4 and t.stride(-1) == 1
-    return ctypes.byref(View4(t.data_ptr(), _stride(t, 0), _stride(t, 1), _stride(t, 2)))
+    (n0, n1, n2, _), (s0, s1, s2, s3) = t.shape, t.stride()      # raises unless t has four dimensions
+    assert s3 == 1
+    # the stride of a dimension of extent 1 is never used; torch leaves arbitrary values there
+    return ctypes.byref(View4(t.data_ptr(), s0 if n0 > 1 else 0, s1 if n1 > 1 else 0, s2 if n2 > 1 else 0))
 
 
 def ptr(t):
@@ -59,8 +56,13 @@ def check(code, what):
 
 
 def is_kernel_ready(t):
-    return (t.stride(-1) == 1 and t.data_ptr() % 16 == 0
-            and all(_stride(t, d) % 8 == 0 for d in range(t.dim() - 1)))
+    strides = t.stride()
+    if strides[-1] != 1 or t.data_ptr() % 16:
+        return False
+    for extent, stride in zip(t.shape[:-1], strides[:-1]):
+        if extent > 1 and stride % 8:
+            return False
+    return True
 
 
 def kernel_ready(t):
