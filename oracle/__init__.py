@@ -24,17 +24,17 @@ randomized three-way comparison), see ``tests/test_oracle_*.py``:
 
 * ``dropout.keep_mask`` (+ the ``dropout_mask`` argument of ``flash_attention``): Philox-4x32 against
   the Random123 known-answer vectors, the uniform map against its defining properties, the drop
-  rate; dropout with an all-true mask equals no dropout; a hand-built mask against an explicit loop.
+  rate, Triton's ``tl.rand`` and the reference's recomputed masks bit for bit; dropout with an all-true
+  mask equals no dropout; a hand-built mask against an explicit loop.
 
 All three operators are also held against fixed vectors (``tests/golden/attention_vectors.npz``, written by
 ``tests/golden/make_vectors.py`` from scalar fp64 loops that state the definitions directly): bottom-right
 causal alignment with grouped heads, rows without keys, the piecewise distance rule, the paged block
 table (``tests/test_golden.py``; the same vectors check the kernels in the simulator and on the GPU).
 
-No function of this oracle is "parity unpinned" with respect to what the kernels are compared
-against.  One statement is: that ``dropout.keep_mask`` reproduces, bit for bit, the mask a Triton run
-of the reference would draw -- it restates Triton's published ``tl.rand`` but no such run is possible
-here (no GPU with Triton), so bitwise mask parity with the reference is unpinned.
+No function of this oracle is "parity unpinned".  ``dropout.keep_mask`` in particular reproduces, bit for
+bit, Triton's ``tl.rand`` and the masks of the reference's ``recompute_mask_kernel`` (run with Triton's CPU
+interpreter; ``tests/golden/dropout_vectors.npz``).
 """
 from .flash import flash_attention  # noqa: F401
 from .piecewise import piecewise_attention, piecewise_attention_grad  # noqa: F401

@@ -13,10 +13,15 @@ with Triton's ``tl.rand(seed, offs, n_rounds=6)`` (dependency ``triton>=2.2.0``,
 algorithm is restated here: Philox-4x32 with multipliers 0xD2511F53 / 0xCD9E8D57 and key increments
 0x9E3779B9 / 0xBB67AE85, and uniform(x) = (x as int32, negative values mapped to -x - 1) * 4.6566127342e-10.
 
-Pinned by: the Random123 known-answer vectors of philox4x32 with 10 rounds (tests/test_oracle_dropout.py;
-the round function does not depend on the round count), the drop rate, and the bounds of the uniform map.
-Bit equality with a Triton run of the reference is not checked (no Triton on a GPU here): parity unpinned
-for that statement only; everything the kernels are compared against is this file.
+Pinned by (tests/test_oracle_dropout.py): the Random123 known-answer vectors of philox4x32 with 10 rounds
+(the round function does not depend on the round count), the drop rate, the bounds of the uniform map --
+and, bit for bit, by what Triton 3.6.0's ``tl.rand`` returns for seeds and counters on both sides of 2^31
+and 2^32 and by the masks the reference's ``recompute_mask_kernel`` draws, both produced with Triton's CPU
+interpreter (tests/golden/make_dropout_vectors.py -> tests/golden/dropout_vectors.npz).
+
+One difference is known and lies outside what the reference can do: its kernels form the counter in 32-bit
+arithmetic whenever seed offset and tensor extents fit 32 bits (Triton types integer arguments by value),
+so it wraps for score tensors of 2^31 elements and more; the counter here is 64 bits wide throughout.
 """
 import numpy as np
 import torch

@@ -1,5 +1,9 @@
 """Pins oracle/dropout.py: Philox-4x32 against the Random123 known-answer vectors, the uniform map
-against its defining properties, and the mask against its drop rate."""
+against its defining properties, the mask against its drop rate -- and both against what Triton's own
+``tl.rand`` and the reference's ``recompute_mask_kernel`` produce (tests/golden/dropout_vectors.npz, written
+by tests/golden/make_dropout_vectors.py with Triton's CPU interpreter)."""
+import os
+
 import numpy as np
 import pytest
 
@@ -75,3 +79,36 @@ def test_flash_oracle_with_dropout_mask():
                 if mask[0, h, m, n]:
                     ref[0, h, m] += p[n] * v[0, h, n] / 0.6
     assert torch.allclose(out, ref, atol=1e-6)
+
+
+GOLDEN = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "dropout_vectors.npz"))
+RAND_CASES = sorted(int(k.split("_")[1]) for k in GOLDEN.files if k.startswith("rand_") and k.endswith("_args"))
+MASK_CASES = sorted(int(k.split("_")[1]) for k in GOLDEN.files if k.startswith("mask_") and k.endswith("_args"))
+
+
+@pytest.mark.parametrize("case", RAND_CASES)
+def test_uniform_numbers_equal_tritons_rand_bit_for_bit(case):
+    """tl.rand(seed, first + arange(count), n_rounds=6) of Triton 3.6.0: seeds and counters on both sides of
+    2^31 and 2^32, so the 32-bit and the 64-bit argument forms are both covered."""
+    seed, first, count = (int(x) for x in GOLDEN[f"rand_{case}_args"])
+    counter = np.uint64(first) + np.arange(count, dtype=np.uint64)
+    zeros = np.zeros(count, dtype=np.uint32)
+    x, _, _, _ = philox4x32((counter & np.uint64(0xFFFFFFFF)).astype(np.uint32), (counter >> np.uint64(32)).astype(np.uint32),
+                            zeros, zeros, seed & 0xFFFFFFFF, seed >> 32, 6)
+    assert np.array_equal(uniform_from_bits(x).view(np.uint32), GOLDEN[f"rand_{case}_values"].view(np.uint32))
+
+
+@pytest.mark.parametrize("case", MASK_CASES)
+def test_mask_equals_the_references_recomputed_mask(case):
+    """recompute_mask_kernel (src/flag_attn/testing/dropout.py:5-17 of the reference) on the same arguments."""
+    B, H, M, N, seed, offset = (int(x) for x in GOLDEN[f"mask_{case}_args"])
+    p = float(GOLDEN[f"mask_{case}_p"])
+    expected = np.unpackbits(GOLDEN[f"mask_{case}_bits"])[:B * H * M * N].astype(bool).reshape(B, H, M, N)
+    assert np.array_equal(keep_mask(B, H, M, N, p, seed, offset).numpy(), expected)
+
+
+def test_the_fixture_covers_both_argument_widths():
+    firsts = [int(GOLDEN[f"rand_{c}_args"][1]) for c in RAND_CASES]
+    seeds = [int(GOLDEN[f"rand_{c}_args"][0]) for c in RAND_CASES]
+    assert min(firsts) < 2 ** 31 < 2 ** 32 < max(firsts) and min(seeds) < 2 ** 31 < 2 ** 32 < max(seeds)
+    assert len(MASK_CASES) >= 4 and str(GOLDEN["triton_version"]) == "3.6.0"
