@@ -61,19 +61,41 @@ def get_bwd_config(B, H, M, N, D, causal):
     return (64, 128, 2, 4)
 
 
+def _check_arguments(q, k, v, dropout_p):
+    """The argument checks of ``flash.py:27-38`` of the reference."""
+    Dq, Dk, Dv = q.shape[-1], k.shape[-1], v.shape[-1]
+    assert Dq == Dk == Dv, "feature size of q, k, v should be equal"
+    assert Dk in _HEAD_DIMS
+    Hk, Hv = k.shape[1], v.shape[1]
+    assert Hk == Hv, "num of heads in k and v should be equal"
+    assert Hk > 0 and q.shape[1] % Hk == 0, "number of heads in q must be a multiple of that in k & v"
+    assert 0.0 <= dropout_p < 1.0, "dropout_p must be in [0, 1)"
+
+
+class NothingToAttend(torch.autograd.Function):
+    """An empty batch, query or key axis: no kernel has anything to do.  A query row without keys gives
+    O = 0 and L = -inf, as rows hidden entirely by the causal mask do (``flash.py:471-474``), and every
+    gradient is zero.  (The reference divides by zero in its split rule for an empty batch or query axis
+    and returns NaN for an empty key axis.)"""
+
+    @staticmethod
+    def forward(ctx, *inputs):
+        ctx.like = [(t.shape, t.dtype, t.device) for t in inputs]
+        return torch.zeros_like(inputs[0])
+
+    @staticmethod
+    def backward(ctx, do):
+        return tuple(torch.zeros(shape, dtype=dtype, device=device) for shape, dtype, device in ctx.like)
+
+
 class FlashAttention(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v, causal, sm_scale, dropout_p, return_log_normalizer,
                 return_total_attention, return_seed_offset):
-        Dq, Dk, Dv = q.shape[-1], k.shape[-1], v.shape[-1]
-        assert Dq == Dk == Dv, "feature size of q, k, v should be equal"
-        assert Dk in _HEAD_DIMS
+        _check_arguments(q, k, v, dropout_p)
         B, H, M, D = q.shape
         N = k.shape[2]
-        Hk, Hv = k.shape[1], v.shape[1]
-        assert Hk == Hv, "num of heads in k and v should be equal"
-        assert H % Hk == 0, "number of heads in q must be a multiple of that in k & v"
-        assert 0.0 <= dropout_p < 1.0, "dropout_p must be in [0, 1)"
+        Hk = k.shape[1]
         if sm_scale is None:
             sm_scale = 1.0 / math.sqrt(D)
 
@@ -238,7 +260,21 @@ def attention(q, k, v, causal=False, sm_scale=None, dropout_p=0.0,
     offset|None)`` -- exactly the reference's convention (``src/flag_attn/flash.py:150-160``).
     ``dropout_p > 0`` drops probabilities with the reference's Philox scheme (seed and offset taken from
     the device's default generator and returned when ``return_seed_offset`` is set); it cannot be
-    combined with a shape that takes the split-KV path, as in the reference.
+    combined with a shape that takes the split-KV path, as in the reference.  With an empty batch, query
+    or key axis nothing is launched: out is zero, the log-normalizer -inf, the total attention zero.
     """
+    if q.numel() == 0 or k.shape[2] == 0:
+        _check_arguments(q, k, v, dropout_p)
+        B, H, M, _ = q.shape
+        o = NothingToAttend.apply(q, k, v)
+        if not (return_log_normalizer or return_total_attention or return_seed_offset):
+            return o
+        seed = offset = None
+        if dropout_p > 0 and return_seed_offset:
+            seed, offset = philox_cuda_seed_offset(0, q.device)      # nothing is drawn
+        return (o,
+                torch.full((B, H, M), -math.inf, dtype=torch.float32, device=q.device) if return_log_normalizer else None,
+                torch.zeros((B, H, k.shape[2]), dtype=torch.float32, device=q.device) if return_total_attention else None,
+                seed, offset)
     return FlashAttention.apply(q, k, v, causal, sm_scale, dropout_p, return_log_normalizer,
                                 return_total_attention, return_seed_offset)

@@ -37,7 +37,8 @@ def attention(query, key_cache, value_cache, context_lens, block_tables, attn_sc
               max_context_len, num_splits=0):
     """query (num_seqs, heads_q, head_size); key_cache / value_cache (num_blocks, heads_kv, block_size,
     head_size) with identical strides; context_lens (num_seqs,) int32; block_tables (num_seqs,
-    max_blocks_per_seq) int32 or int64.  Returns out shaped like ``query``."""
+    max_blocks_per_seq) int32 or int64.  Returns out shaped like ``query``; a sequence of context length
+    0 gets a zero row."""
     num_seqs, num_q_heads, head_size = query.shape
     num_kv_heads, block_size = key_cache.shape[1], key_cache.shape[2]
     assert key_cache.shape[3] == head_size and value_cache.shape == key_cache.shape
@@ -46,6 +47,8 @@ def attention(query, key_cache, value_cache, context_lens, block_tables, attn_sc
     assert key_cache.stride() == value_cache.stride(), "key and value cache must share their strides"
     assert context_lens.dtype == torch.int32
 
+    if num_seqs == 0:      # nothing to launch
+        return torch.empty(query.shape, dtype=query.dtype, device=query.device)
     lib = _lib.get()
     if query.stride(-1) != 1 or query.data_ptr() % 16 or query.stride(0) % 8 or query.stride(1) % 8:
         query = query.contiguous()

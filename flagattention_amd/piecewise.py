@@ -9,7 +9,7 @@ import math
 import torch
 
 from . import _abi, _config, _lib
-from .flash import _ds_workspace, ds_heads_per_launch
+from .flash import NothingToAttend, _ds_workspace, ds_heads_per_launch
 
 __all__ = ["attention"]
 
@@ -100,5 +100,8 @@ def attention(q1, k1, q2, k2, v, dist_threshold, causal=False, sm_scale=None):
     q1, q2 (batch, heads, seqlen_q, headdim); k1, k2, v (batch, heads, seqlen_k, headdim).  The score
     of query m and key n is ``q2[m].k2[n]`` when the signed distance ``m + seqlen_k - seqlen_q - n``
     is at least ``dist_threshold`` and ``q1[m].k1[n]`` otherwise.  Returns out (batch, heads,
-    seqlen_q, headdim)."""
+    seqlen_q, headdim); zero when the batch, query or key axis is empty (nothing is launched)."""
+    if q1.numel() == 0 or k1.shape[2] == 0:
+        assert q1.shape == q2.shape and k1.shape == k2.shape == v.shape and q1.shape[-1] == k1.shape[-1]
+        return NothingToAttend.apply(q1, k1, q2, k2, v)
     return PiecewiseAttention.apply(q1, k1, q2, k2, v, dist_threshold, causal, sm_scale)

@@ -124,6 +124,8 @@ def attention(q, k, v, causal=False, sm_scale=None):
     Hk, Hv = k.shape[1], v.shape[1]
     assert Hk == Hv, "num of heads in k and v should be equal"
     assert H % Hk == 0, "number of heads in q must be a multiple of that in k & v"
+    if q.numel() == 0 or N == 0:      # nothing to launch; a row without keys is zero
+        return torch.zeros(q.shape, dtype=q.dtype, device=q.device)
     if sm_scale is None:
         sm_scale = 1.0 / math.sqrt(D)
     lib = _lib.get()

@@ -226,3 +226,51 @@ def test_bench_counts_the_flops_of_the_quoted_workloads():
     x2 = 2.0 * c2["B"] * c2["H"] * bench.causal_pairs(c2["T"], c2["T"]) * c2["D"]
     assert abs(7 * x2 / 1e9 - 240.6) < 0.2
     assert bench.PEAK_BF16_TFLOPS == 2500.0 and bench.PEAK_HBM_GBS == 8000.0
+
+
+@pytest.mark.parametrize("B,H,M,N", [(0, 2, 5, 7), (1, 2, 0, 7), (1, 2, 5, 0), (0, 2, 0, 0)])
+def test_empty_axes_launch_nothing(monkeypatch, B, H, M, N):
+    """An empty batch, query or key axis: zero output, -inf log-normalizer, zero total attention and zero
+    gradients of the inputs' shapes, without touching the kernel library.  (The reference's split rule divides
+    by zero for an empty batch or query axis, and its kernels return NaN for an empty key axis.)"""
+    import flag_attn
+    from flagattention_amd import _lib
+
+    def no_library():
+        raise AssertionError("the kernel library must not be needed")
+
+    monkeypatch.setattr(_lib, "get", no_library)
+    D = 32
+    q = torch.randn(B, H, M, D, dtype=torch.float16, requires_grad=True)
+    k = torch.randn(B, 1, N, D, dtype=torch.float16, requires_grad=True)
+    v = torch.randn(B, 1, N, D, dtype=torch.float16, requires_grad=True)
+    o, L, tot, seed, offset = flag_attn.flash_attention(q, k, v, causal=True, return_log_normalizer=True,
+                                                        return_total_attention=True)
+    assert o.shape == q.shape and o.dtype == q.dtype and not o.any()
+    assert L.shape == (B, H, M) and bool((L == -math.inf).all()) and tot.shape == (B, H, N) and not tot.any()
+    assert seed is None and offset is None
+    grads = torch.autograd.grad(o, (q, k, v), torch.ones_like(o))
+    assert [g.shape for g in grads] == [q.shape, k.shape, v.shape] and not any(g.any() for g in grads)
+    assert flag_attn.flash_attention(q, k, v).shape == q.shape
+    assert flag_attn.flash_attention_split_kv(q.detach(), k.detach(), v.detach()).shape == q.shape
+
+    k1 = torch.randn(B, H, N, D, dtype=torch.float16, requires_grad=True)
+    ins = [q, k1, q.detach().clone().requires_grad_(), k1.detach().clone().requires_grad_(), k1.detach().clone().requires_grad_()]
+    o = flag_attn.piecewise_attention(*ins, 3, causal=True)
+    assert o.shape == q.shape and not o.any()
+    grads = torch.autograd.grad(o, ins, torch.ones_like(o))
+    assert [g.shape for g in grads] == [t.shape for t in ins] and not any(g.any() for g in grads)
+
+    with pytest.raises(AssertionError):       # the argument checks still apply
+        flag_attn.flash_attention(q, k, torch.randn(B, 1, N, 2 * D, dtype=torch.float16))
+
+
+def test_paged_attention_without_sequences_launches_nothing(monkeypatch):
+    import flag_attn
+    from flagattention_amd import _lib
+    monkeypatch.setattr(_lib, "get", lambda: (_ for _ in ()).throw(AssertionError("the kernel library must not be needed")))
+    q = torch.empty(0, 8, 64, dtype=torch.float16)
+    cache = torch.empty(4, 2, 16, 64, dtype=torch.float16)
+    out = flag_attn.paged_attention(q, cache, cache, torch.empty(0, dtype=torch.int32),
+                                    torch.empty(0, 4, dtype=torch.int32), 0.125, 0)
+    assert out.shape == q.shape and out.dtype == q.dtype

@@ -12,7 +12,7 @@ import pytest
 import torch
 
 import flag_attn
-from flagattention_amd import _lib, flash, piecewise
+from flagattention_amd import _lib, flash, paged, piecewise
 from oracle import flash_attention as oracle_flash, paged_attention as oracle_paged, piecewise_attention as oracle_pw
 from oracle import within_two_x
 from tests.sim import simlib
@@ -163,3 +163,22 @@ def test_paged_attention_public_call():
     out = flag_attn.paged_attention(q, kc, vc, ctx, table, scale, int(ctx.max()))
     ref = oracle_paged(q.float(), kc.float(), vc.float(), table, ctx, scale)
     assert torch.allclose(out.float(), ref, atol=2e-3, rtol=1e-5)   # tests/flag_attn/test_paged_attention.py:62
+
+
+@pytest.mark.parametrize("launch", [("balanced", 3), ("single", 0), ("partitioned", 2)])
+def test_paged_attention_zero_length_contexts(monkeypatch, launch):
+    """A sequence without keys gets a zero row in every launch form, and does not disturb its neighbours."""
+    seqs, Hq, Hkv, D, bs = 4, 4, 2, 64, 16
+    ctx = torch.tensor([0, 100, 0, 33], dtype=torch.int32)
+    num_blocks = 24
+    table = torch.randint(0, num_blocks, (seqs, 8), dtype=torch.int32, generator=torch.Generator().manual_seed(3))
+    q = rnd(seqs, Hq, D, dtype=torch.float16)
+    kc, vc = rnd(num_blocks, Hkv, bs, D, dtype=torch.float16), rnd(num_blocks, Hkv, bs, D, dtype=torch.float16)
+    num_splits = launch[1] if launch[0] == "partitioned" else 0
+    if launch[0] != "partitioned":
+        monkeypatch.setattr(paged, "choose_launch", lambda *a: launch)
+    out = flag_attn.paged_attention(q, kc, vc, ctx, table, D ** -0.5, 100, num_splits)
+    live = ctx > 0
+    assert not out[~live].any()
+    ref = oracle_paged(q[live].float(), kc.float(), vc.float(), table[live], ctx[live], D ** -0.5)
+    assert torch.allclose(out[live].float(), ref, atol=2e-3, rtol=1e-5)
