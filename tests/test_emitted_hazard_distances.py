@@ -283,7 +283,7 @@ def _audit(obj, tmp_path):
 HAND_SLOTTED = ("fa_fwd_wide_kernel", "fa_bwd_dkdv_kernel")
 
 
-@pytest.mark.parametrize("obj", ["fa_fwd_wide.o", "fa_bwd.o", "fa_fwd.o", "fa_splitkv.o", "fa_total.o"])
+@pytest.mark.parametrize("obj", ["fa_fwd_wide.o", "fa_bwd.o", "fa_fwd.o", "fa_splitkv.o", "fa_total.o", "paged.o"])
 def test_vector_accesses_to_matrix_results_keep_their_distance(obj, tmp_path):
     """Reads everywhere; overwrites in the hand-slotted kernels.  (In compiler-scheduled code a few overwrites that
     are reached only over a taken skip branch count fewer wait states than the compiler pads to elsewhere; that
