@@ -11,6 +11,9 @@
  * (batch, head, token, D) view whose D stride is 1.  Pointers must be 16-byte aligned and the three
  * strides multiples of 8 elements.  `dtype` is FA_F16 or FA_BF16 and applies to every 16-bit tensor
  * of the call; log-normalizer, delta, total-attention and partial-softmax buffers are fp32.
+ * Batch, head and query extents must be positive and pointers non-null (FA_ERR_BAD_ARGUMENT
+ * otherwise): a caller with an empty problem launches nothing.  A paged sequence of context length 0
+ * is valid and gets a zero output row.
  *
  * Each declaration cites the interface of the reference (FlagOpen/FlagAttention, Triton) that it
  * replaces.
