@@ -208,8 +208,12 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (D <= 128 ? 2 : 1)) paged_balanced_ke
   for (int base = 0; base < p.num_seqs; base += 64) {
     const int s = base + lane;
     const int u = s < p.num_seqs ? units_of(s) : 0;
-    if (w == 0 && tid < 64 && s < p.num_seqs && u == 0) {  // an empty sequence has no keys to stream: its output rows are zero
-      for (int i = 0; i < p.Hq * D; ++i) ((T*)p.out)[(int64_t)s * p.o_ss + (int64_t)(i / D) * p.o_sh + i % D] = (T)0.f;
+    // An empty sequence has no keys to stream: its output rows are zero.  Every wavefront sees the same
+    // empty sequences here; they are dealt round-robin to the workgroups, and the threads of the one
+    // that takes a sequence clear its rows together.
+    for (uint64_t todo = hw::ballot(s < p.num_seqs && u == 0 && s % p.num_wgs == w); todo; todo &= todo - 1) {
+      const int e = base + __builtin_ctzll(todo);
+      for (int i = tid; i < p.Hq * D; i += kThreads) ((T*)p.out)[(int64_t)e * p.o_ss + (int64_t)(i / D) * p.o_sh + i % D] = (T)0.f;
     }
     total_units += hw::uniform(hw::lane_value(prefix_in_wave(u), 63));
   }

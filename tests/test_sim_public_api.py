@@ -182,3 +182,26 @@ def test_paged_attention_zero_length_contexts(monkeypatch, launch):
     assert not out[~live].any()
     ref = oracle_paged(q[live].float(), kc.float(), vc.float(), table[live], ctx[live], D ** -0.5)
     assert torch.allclose(out[live].float(), ref, atol=2e-3, rtol=1e-5)
+
+
+@pytest.mark.parametrize("num_wgs", [1, 7, 40])
+def test_paged_attention_many_empty_sequences(monkeypatch, num_wgs):
+    """Empty sequences are dealt round-robin to the workgroups of the balanced launch, also to those that
+    have no keys to stream; more sequences than one scan step (64) and than workgroups."""
+    seqs, Hq, Hkv, D, bs = 130, 4, 2, 32, 16
+    gen = torch.Generator().manual_seed(11)
+    ctx = torch.zeros(seqs, dtype=torch.int32)
+    live_at = [0, 63, 64, 97, 129]
+    ctx[live_at] = torch.tensor([5, 130, 1, 40, 77], dtype=torch.int32)
+    num_blocks = 32
+    table = torch.randint(0, num_blocks, (seqs, 9), dtype=torch.int32, generator=gen)
+    q = rnd(seqs, Hq, D, dtype=torch.float16)
+    kc, vc = rnd(num_blocks, Hkv, bs, D, dtype=torch.float16), rnd(num_blocks, Hkv, bs, D, dtype=torch.float16)
+    monkeypatch.setattr(paged, "choose_launch", lambda *a: ("balanced", num_wgs))
+    real_empty = torch.empty
+    monkeypatch.setattr(torch, "empty", lambda *a, **kw: real_empty(*a, **kw).fill_(7) if kw.get("dtype") == q.dtype else real_empty(*a, **kw))
+    out = flag_attn.paged_attention(q, kc, vc, ctx, table, D ** -0.5, 130)
+    live = ctx > 0
+    assert not out[~live].any()          # the output buffer started out as sevens
+    ref = oracle_paged(q[live].float(), kc.float(), vc.float(), table[live], ctx[live], D ** -0.5)
+    assert torch.allclose(out[live].float(), ref, atol=2e-3, rtol=1e-5)
