@@ -4,7 +4,9 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2]
 
 A step is one forward + backward pass of ``flash_attention`` (public API, autograd) over one batch
-of synthetic bf16 inputs that already sit in HBM.  Default workload: causal, B=1, H=32, T=8192,
+of synthetic bf16 inputs that already sit in HBM.  Before the W warm-up steps the same step runs untimed
+for ``--prewarm-seconds`` (default 0.5 s), so that the K timed steps see the clocks of a loaded device
+rather than the ramp from idle.  Default workload: causal, B=1, H=32, T=8192,
 D=128 -- the configuration the target of the metric is quoted on.  ``value`` counts matmul-only
 FLOPs with the reference's convention (benchmark/flash_benchmark.py:95-103 of the reference):
 forward 4*B*H*M*N*D, backward 2.5x that, halved under the causal mask.
@@ -117,6 +119,15 @@ def flash_step_bench(args, torch):
         o = flag_attn.flash_attention(q, k, v, causal=True, sm_scale=sm_scale)
         return torch.autograd.grad(o, (q, k, v), do)
 
+    # Untimed pre-warm by time, not by count: the step loop is the first GPU work of the process, and a device
+    # that starts from its idle clocks takes about 100 ms of continuous load to settle (a kernel trace of the
+    # cold loop shows back-to-back launches with no gaps whose durations fall by 15-30 % over the first 40
+    # steps: profiles/step_loop_cold_start_kernel_trace.txt).  --warmup steps follow, then the timed steps.
+    t_warm = time.perf_counter()
+    while time.perf_counter() - t_warm < args.prewarm_seconds:
+        for _ in range(5):
+            step()
+        torch.cuda.synchronize()
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -180,7 +191,8 @@ def flash_step_bench(args, torch):
 
 
 def cpu_baseline(args, torch):
-    """The fp32 oracle on the host cores over a bounded sample: 2 of the workload's heads."""
+    """The fp32 oracle on the host cores over a bounded sample: 8 of the 32 heads at T = 8192 (all 32 of the
+    batch-1 slice at T = 2048)."""
     from oracle import flash_attention
     w = WORKLOADS[args.workload]
     T, D = w["T"], w["D"]
@@ -368,6 +380,8 @@ def main():
     ap.add_argument("--hold-seconds", type=float, default=0.0,
                     help="with --profile-kernel: afterwards repeat the launch for this long")
     ap.add_argument("--no-paged", action="store_true")
+    ap.add_argument("--prewarm-seconds", type=float, default=0.5,
+                    help="untimed steps run for this long before the counted --warmup steps (0 = none)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (every (batch, head) slice "

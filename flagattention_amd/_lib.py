@@ -46,11 +46,13 @@ SIGNATURES = {
     "paged_attn_balanced_workspace": [_i, _i],
     "paged_attn_balanced": [_i, _p, _i64, _i64, _p, _i64, _i64, _p, _p, _i64, _i64, _i64, _p, _p, _i, _i64,
                             _f, _i, _i, _i, _i, _i, _p, _i64, _i, _p],
+    "paged_attn_balanced_static_prepare": [],
     "paged_attn_balanced_static": [_i, _p, _i64, _i64, _p, _i64, _i64, _p, _p, _i64, _i64, _i64, _p, _p, _i, _i64,
                                    _f, _i, _i, _i, _i, _i, _i, _p],
 }
 
 STATIC_SCRATCH_BYTES = 17 * 1024 * 1024   # FA_STATIC_SCRATCH_BYTES of include/flagattn.h
+ABI_VERSION = 2                           # FA_ABI_VERSION of include/flagattn.h: the revision SIGNATURES describes
 
 
 def bind(path, names=None):
@@ -62,6 +64,11 @@ def bind(path, names=None):
         fn = getattr(lib, name)  # AttributeError if the library lacks a declared symbol
         fn.argtypes = argtypes
         fn.restype = ctypes.c_int
+    if names is None or "fa_version" in names:
+        built = lib.fa_version()
+        if built != ABI_VERSION:
+            raise RuntimeError(f"{path} implements revision {built} of the C interface, this package binds "
+                               f"revision {ABI_VERSION}: rebuild the library (`make -C flagattention_amd/csrc`)")
     return lib
 
 

@@ -8,7 +8,7 @@
 
 namespace {
 
-constexpr int kVersion = 1;
+constexpr int kVersion = FA_ABI_VERSION;
 
 bool head_dim_ok(int D) { return D == 16 || D == 32 || D == 64 || D == 128; }
 
@@ -29,15 +29,29 @@ fa::View4 to_view(const fa_view4* v) {
 
 }  // namespace
 
+namespace fa {
+int num_cus_of_current_device() {
+  constexpr int kDevices = 64;
+  static std::atomic<int> known[kDevices];
+  int dev = -1, n = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0) return 0;
+  if (dev < kDevices) {
+    n = known[dev].load(std::memory_order_relaxed);
+    if (n > 0) return n;
+  }
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 0;
+  if (dev < kDevices) known[dev].store(n, std::memory_order_relaxed);
+  return n;
+}
+}  // namespace fa
+
 extern "C" {
 
 int fa_version(void) { return kVersion; }
 
 int fa_num_cus(void) {
-  int dev = 0, n = 0;
-  if (hipGetDevice(&dev) != hipSuccess) return -1;
-  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return -1;
-  return n;
+  const int n = fa::num_cus_of_current_device();
+  return n > 0 ? n : -1;
 }
 
 int fa_fwd(int dtype, const fa_view4* q, const fa_view4* k, const fa_view4* v, const fa_view4* o,
@@ -388,6 +402,11 @@ int scratch_of_current_device(void** out) {
   return 0;
 }
 }  // namespace
+
+int paged_attn_balanced_static_prepare(void) {
+  void* ws = nullptr;
+  return scratch_of_current_device(&ws);
+}
 
 int paged_attn_balanced_static(int dtype, void* out, int64_t o_stride_s, int64_t o_stride_h, const void* query,
                                int64_t q_stride_s, int64_t q_stride_h, const void* key_cache,

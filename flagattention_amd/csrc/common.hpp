@@ -6,7 +6,10 @@
 //   * one wavefront multiplies 32x32 blocks with mfma32 (hw.hpp); its lane l owns column l % 32 of a
 //     block and the half h = l / 32 selects which rows / which 8 of the 16 contraction indices.
 #pragma once
+#include <atomic>
+#include <mutex>
 #include <type_traits>
+#include <unordered_map>
 #include <utility>
 
 #include "hw.hpp"
@@ -194,12 +197,37 @@ FA_DEVICE bool dropout_keeps(uint64_t counter, uint64_t seed, float dropout_p) {
 // ---------------------------------------------------------------------------------------------
 // launch
 // ---------------------------------------------------------------------------------------------
+constexpr int kMaxDevices = 64;   // devices whose per-device facts are remembered
+
+// A kernel that needs more than 48 KB of LDS has to be given the limit before its first launch, once per
+// device (the attribute belongs to the device's copy of the function).  The runtime call costs about as
+// much as a launch, so the devices on which it has been made are remembered per kernel.
+template <class P>
+int allow_lds(void (*kern)(P), size_t lds_bytes) {
+  static std::mutex lock;
+  static std::unordered_map<const void*, uint64_t> done;   // kernel -> bit per device
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0) dev = kMaxDevices;
+  const uint64_t bit = dev < kMaxDevices ? (uint64_t)1 << dev : 0;
+  if (bit) {
+    std::lock_guard<std::mutex> g(lock);
+    auto it = done.find((const void*)kern);
+    if (it != done.end() && (it->second & bit)) return 0;
+  }
+  hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+  if (e != hipSuccess) return (int)e;
+  if (bit) {
+    std::lock_guard<std::mutex> g(lock);
+    done[(const void*)kern] |= bit;
+  }
+  return 0;
+}
+
 template <class P>
 int launch(void (*kern)(P), dim3 grid, size_t lds_bytes, hipStream_t stream, const P& p) {
   if (lds_bytes > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)lds_bytes);
-    if (e != hipSuccess) return (int)e;
+    const int rc = allow_lds(kern, lds_bytes);
+    if (rc) return rc;
   }
   hipLaunchKernelGGL(kern, grid, dim3(kThreads), lds_bytes, stream, p);
   return (int)hipGetLastError();

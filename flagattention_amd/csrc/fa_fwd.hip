@@ -274,13 +274,8 @@ static int dispatch_fwd(const FwdParams& p, bool piecewise, hipStream_t stream) 
 // Which kernel a launch without an explicit tile takes: the 256-row kernel is the faster one per tile,
 // but its workgroups hold a compute unit alone, so it needs at least one workgroup per compute unit.
 static bool prefer_wide(const FwdParams& p) {
-  static int num_cus = 0;   // one device kind per process
-  if (num_cus == 0) {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return false;
-    num_cus = n;
-  }
-  return (int64_t)((p.M + 255) / 256) * p.H * p.B >= num_cus;
+  const int num_cus = num_cus_of_current_device();
+  return num_cus > 0 && (int64_t)((p.M + 255) / 256) * p.H * p.B >= num_cus;
 }
 
 int run_fwd(const FwdParams& p, bool piecewise, hipStream_t stream) {

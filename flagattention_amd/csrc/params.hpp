@@ -61,6 +61,8 @@ struct TotalParams {
 #include "hw.hpp"  // hipStream_t
 
 namespace fa {
+// Compute units of the current device (0 if the runtime cannot tell); asked once per device, then remembered.
+int num_cus_of_current_device();
 int run_fwd(const FwdParams& p, bool piecewise, hipStream_t stream);
 bool fwd_wide_supported(const FwdParams& p);   // the 256-row kernel (fa_fwd_wide.hip) can serve this launch
 int run_fwd_wide(const FwdParams& p, hipStream_t stream);

@@ -55,6 +55,9 @@ def _num_cus():
     return _NUM_CUS[dev]
 
 
+_DEFAULT_FWD_CONFIG = get_fwd_config
+
+
 def get_bwd_config(B, H, M, N, D, causal):
     """(BLOCK_M, BLOCK_N, num_stages, num_warps) of the dK/dV kernel: queries per pipeline step, keys
     per workgroup (``flash.py:493-519`` hook, called as in ``flash.py:185-186``; see ``BWD_TILES``)."""
@@ -103,7 +106,7 @@ class FlashAttention(torch.autograd.Function):
         q, k, v = _abi.kernel_ready(q), _abi.kernel_ready(k), _abi.kernel_ready(v)
 
         with torch.cuda.device(q.device):
-            num_cus = lib.fa_num_cus()
+            num_cus = _num_cus()
             is_dropout = dropout_p > 0
             if is_dropout:   # one Philox counter value per score element (flash.py:52-57)
                 seed, offset = philox_cuda_seed_offset(B * H * M * N, q.device)
@@ -118,12 +121,26 @@ class FlashAttention(torch.autograd.Function):
                 o, L = split_kv_forward(lib, q, k, v, causal, sm_scale, splits)
             else:
                 # looked up by name at call time, so that an assignment to flash.get_fwd_config takes effect
-                block_m, _ = _config.resolve(get_fwd_config, FWD_TILES, "flash_attention forward",
-                                             (B, H, M, N, D, causal))
-                if block_m == 256 and not (wide_forward_applies(D, dropout_p) and sm_scale > 0):
+                hook = get_fwd_config
+                block_m, _ = _config.resolve(hook, FWD_TILES, "flash_attention forward", (B, H, M, N, D, causal))
+                if hook is _DEFAULT_FWD_CONFIG:
+                    # nobody overrode the hook: the library applies the same rule and also knows what the hook
+                    # is not told (dropout, the sign of sm_scale, row strides the 256-row kernel cannot address)
+                    block_m = 0
+                elif block_m == 256 and not wide_forward_applies(D, dropout_p):
                     _config.warn_once(("fwd-wide", D, is_dropout),
                                       "flash_attention forward: the 256-row kernel is built for head size 128 "
                                       "without dropout; launching the 128-row kernel")
+                    block_m = 128
+                elif block_m == 256 and not sm_scale > 0:
+                    _config.warn_once(("fwd-wide-scale",),
+                                      "flash_attention forward: the 256-row kernel needs sm_scale > 0; launching "
+                                      "the 128-row kernel")
+                    block_m = 128
+                elif block_m == 256 and max(k.stride(2), v.stride(2)) * k.element_size() >= 1 << 24:
+                    _config.warn_once(("fwd-wide-stride",),
+                                      "flash_attention forward: the 256-row kernel addresses key/value rows less "
+                                      "than 16 MiB apart; launching the 128-row kernel")
                     block_m = 128
                 o = torch.empty_like(q)
                 if not _abi.is_kernel_ready(o):
@@ -163,7 +180,7 @@ class FlashAttention(torch.autograd.Function):
             # dK/dV come out summed over each kv head's group of query heads (flash.py:205-206,250-251
             # of the reference produce one slice per query head and reduce afterwards)
             # the kernels that sum query heads are built without dropout
-            chunk = 1 if dropout[0] > 0 else dkdv_heads_per_slice(B, H, group, N, lib.fa_num_cus())
+            chunk = 1 if dropout[0] > 0 else dkdv_heads_per_slice(B, H, group, N, _num_cus())
             slices = H // chunk
             dk = torch.empty((B, slices, N, D), dtype=k.dtype, device=q.device)
             dv = torch.empty((B, slices, N, D), dtype=v.dtype, device=q.device)

@@ -33,10 +33,21 @@ def choose_launch(num_seqs, num_kv_heads, group, head_size, max_context_len, num
     return "balanced", num_wgs
 
 
+_NUM_CUS = {}
+
+
+def _num_cus(lib, device):
+    """Compute units of ``device`` (asked once; the current device is ``device`` when this is called)."""
+    key = (device.index if device.index is not None else torch.cuda.current_device()) if device.type == "cuda" else -1
+    if key not in _NUM_CUS:
+        _NUM_CUS[key] = lib.fa_num_cus()
+    return _NUM_CUS[key]
+
+
 def attention(query, key_cache, value_cache, context_lens, block_tables, attn_scale,
               max_context_len, num_splits=0):
     """query (num_seqs, heads_q, head_size); key_cache / value_cache (num_blocks, heads_kv, block_size,
-    head_size) with identical strides; context_lens (num_seqs,) int32; block_tables (num_seqs,
+    head_size) with identical strides; context_lens (num_seqs,) of any integer type; block_tables (num_seqs,
     max_blocks_per_seq) int32 or int64.  Returns out shaped like ``query``; a sequence of context length
     0 gets a zero row."""
     num_seqs, num_q_heads, head_size = query.shape
@@ -45,24 +56,29 @@ def attention(query, key_cache, value_cache, context_lens, block_tables, attn_sc
     assert head_size in _HEAD_SIZES, f"head_size={head_size}"
     assert num_q_heads % num_kv_heads == 0
     assert key_cache.stride() == value_cache.stride(), "key and value cache must share their strides"
-    assert context_lens.dtype == torch.int32
+    assert not context_lens.dtype.is_floating_point and context_lens.dtype != torch.bool, \
+        f"context_lens must hold integers, got {context_lens.dtype}"
 
     if num_seqs == 0:      # nothing to launch
-        return torch.empty(query.shape, dtype=query.dtype, device=query.device)
+        return torch.empty_like(query)
     lib = _lib.get()
     if query.stride(-1) != 1 or query.data_ptr() % 16 or query.stride(0) % 8 or query.stride(1) % 8:
         query = query.contiguous()
     assert key_cache.stride(-1) == 1
+    if context_lens.dtype != torch.int32:   # the kernels read 32-bit lengths (the reference takes any integer type)
+        context_lens = context_lens.to(torch.int32)
     context_lens = context_lens.contiguous()
     if block_tables.stride(-1) != 1:
         block_tables = block_tables.contiguous()
-    out = torch.empty(query.shape, dtype=query.dtype, device=query.device)
+    out = torch.empty_like(query)   # the caller's layout, as paged.py:16 of the reference, when the kernels can write it
+    if out.stride(-1) != 1 or out.data_ptr() % 16 or out.stride(0) % 8 or out.stride(1) % 8:
+        out = torch.empty(query.shape, dtype=query.dtype, device=query.device)
     group = num_q_heads // num_kv_heads
 
     with torch.cuda.device(query.device):
         if num_splits == 0:
             kind, num_wgs = choose_launch(num_seqs, num_kv_heads, group, head_size, max_context_len,
-                                          lib.fa_num_cus())
+                                          _num_cus(lib, query.device))
             if kind == "balanced":
                 nbytes = lib.paged_attn_balanced_workspace(num_wgs, head_size)
                 workspace = torch.empty(nbytes // 4, dtype=torch.float32, device=query.device)

@@ -36,6 +36,8 @@ def total_attention(q, k, l, causal=False, sm_scale=None):
     assert q.shape[1] % k.shape[1] == 0, "number of heads in q must be a multiple of that in k"
     if sm_scale is None:
         sm_scale = 1.0 / math.sqrt(Dq)
+    if q.numel() == 0 or k.shape[2] == 0:   # an empty batch, query or key axis: nothing attends to anything
+        return torch.zeros((q.shape[0], q.shape[1], k.shape[2]), dtype=torch.float32, device=q.device)
     lib = _lib.get()
     q, k = _abi.kernel_ready(q), _abi.kernel_ready(k)
     l = l.contiguous()

@@ -39,7 +39,10 @@ typedef struct fa_view4 {
   int64_t stride_b, stride_h, stride_t; /* in elements */
 } fa_view4;
 
-/* Library facts. */
+/* Library facts.  fa_version() returns the FA_ABI_VERSION the library was built from; it changes whenever an
+ * entry point changes its argument list (2: fa_fwd gained block_m), and a caller built against another
+ * revision must not call the library. */
+#define FA_ABI_VERSION 2
 int fa_version(void);
 /* Number of compute units of the current device (the reference reads
  * torch.cuda.get_device_properties(...).multi_processor_count, src/flag_attn/flash.py:47-48). */
@@ -223,7 +226,9 @@ int paged_attn_balanced(int dtype, void* out, int64_t o_stride_s, int64_t o_stri
  * paged.py:92-108).  Same arguments and same result as paged_attn_balanced minus the workspace: the
  * partial-result slots live in a device array of FA_STATIC_SCRATCH_BYTES inside the library, which
  * every device that runs the library holds until the process ends.  The call allocates and frees
- * nothing (the array's device address is looked up on the first call on each device).  A launch whose
+ * nothing.  The array's device address is looked up on the first call on each device, which makes the
+ * runtime load the library's code object there: that first call (or paged_attn_balanced_static_prepare(),
+ * which does the lookup and launches nothing) has to happen before a stream capture begins.  A launch whose
  * paged_attn_balanced_workspace(num_workgroups, head_size) exceeds FA_STATIC_SCRATCH_BYTES is rejected
  * with FA_ERR_SCRATCH_TOO_SMALL and nothing is launched (the array holds 1024 workgroups at head_size
  * <= 128 and 256 workgroups at head_size 512: more than one resident wave of a 256-CU device).  All calls on
@@ -231,6 +236,9 @@ int paged_attn_balanced(int dtype, void* out, int64_t o_stride_s, int64_t o_stri
  * that do not order their launches) race on it and must use paged_attn_balanced with separate
  * workspaces instead. */
 #define FA_STATIC_SCRATCH_BYTES (17 * 1024 * 1024)
+/* Looks up (and remembers) the scratch array's address on the current device; launches nothing.  Returns 0,
+ * or the runtime's error.  Like paged_attn_balanced_static it has no counterpart in the reference. */
+int paged_attn_balanced_static_prepare(void);
 int paged_attn_balanced_static(int dtype, void* out, int64_t o_stride_s, int64_t o_stride_h, const void* query,
                                int64_t q_stride_s, int64_t q_stride_h, const void* key_cache,
                                const void* value_cache, int64_t kv_stride_blk, int64_t kv_stride_h,

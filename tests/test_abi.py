@@ -40,7 +40,18 @@ def test_library_exports_every_declared_symbol():
     if not os.path.exists(_lib.LIB_PATH):
         pytest.fail(f"{_lib.LIB_PATH} has not been built (run `python -c 'import __graft_entry__ as g; g.build()'`)")
     lib = _lib.bind(_lib.LIB_PATH)  # getattr on every declared name; raises if one is missing
-    assert lib.fa_version() >= 1
+    assert lib.fa_version() == _lib.ABI_VERSION
+    text = open(HEADER).read()
+    assert int(re.search(r"#define\s+FA_ABI_VERSION\s+(\d+)", text).group(1)) == _lib.ABI_VERSION
+
+
+def test_loader_refuses_a_library_of_another_interface_revision(monkeypatch):
+    """A caller built against another argument list must not call the library: bind() compares revisions."""
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.fail(f"{_lib.LIB_PATH} has not been built")
+    monkeypatch.setattr(_lib, "ABI_VERSION", _lib.ABI_VERSION + 1)
+    with pytest.raises(RuntimeError, match="revision"):
+        _lib.bind(_lib.LIB_PATH)
 
 
 def test_missing_library_raises(monkeypatch, tmp_path):

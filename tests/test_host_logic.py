@@ -274,3 +274,85 @@ def test_paged_attention_without_sequences_launches_nothing(monkeypatch):
     out = flag_attn.paged_attention(q, cache, cache, torch.empty(0, dtype=torch.int32),
                                     torch.empty(0, 4, dtype=torch.int32), 0.125, 0)
     assert out.shape == q.shape and out.dtype == q.dtype
+
+
+def test_total_attention_with_empty_axes_launches_nothing(monkeypatch):
+    """The standalone total_attention treats an empty batch, query or key axis like flash_attention does."""
+    import flag_attn
+    from flagattention_amd import _lib
+    monkeypatch.setattr(_lib, "get", lambda: (_ for _ in ()).throw(AssertionError("the kernel library must not be needed")))
+    for B, H, M, N in [(0, 2, 5, 7), (1, 2, 0, 7), (1, 2, 5, 0)]:
+        q = torch.randn(B, H, M, 32, dtype=torch.float16)
+        k = torch.randn(B, 1, N, 32, dtype=torch.float16)
+        tot = flag_attn.total_attention(q, k, torch.zeros(B, H, M), causal=True)
+        assert tot.shape == (B, H, N) and tot.dtype == torch.float32 and not tot.any()
+
+
+class _RecordingLibrary:
+    """Stands in for the kernel library: every entry point returns 0 and is recorded with its arguments."""
+
+    def __init__(self):
+        self.calls = []
+
+    def __getattr__(self, name):
+        if name == "fa_num_cus":
+            return lambda: 256
+        if name == "paged_attn_balanced_workspace":
+            return lambda wgs, d: 1024
+
+        def call(*args):
+            self.calls.append((name, args))
+            return 0
+        return call
+
+
+def _with_recording_library(monkeypatch):
+    import contextlib
+    from flagattention_amd import _lib, flash, paged
+    lib = _RecordingLibrary()
+    monkeypatch.setattr(_lib, "get", lambda: lib)
+    monkeypatch.setattr(torch.cuda, "device", lambda device: contextlib.nullcontext())
+    monkeypatch.setattr(flash, "_NUM_CUS", {})
+    monkeypatch.setattr(paged, "_NUM_CUS", {})
+    return lib
+
+
+def test_default_forward_hook_leaves_the_tile_to_the_library(monkeypatch, recwarn):
+    """With the module's own get_fwd_config nobody chose a tile: fa_fwd gets block_m = 0, so that a large head-128
+    launch with dropout (which the hook is not told about) warns about nothing, and so does a stride the
+    256-row kernel cannot address; an override that asks for 256 rows where they do not apply is told once."""
+    import flag_attn
+    from flagattention_amd import flash, _config
+    lib = _with_recording_library(monkeypatch)
+    monkeypatch.setattr(flash, "philox_cuda_seed_offset", lambda n, device: (1, 2))
+    monkeypatch.setattr(_config, "_warned", set())
+    q = torch.empty(1, 32, 8192, 128, dtype=torch.bfloat16)
+    assert flash.get_fwd_config(1, 32, 8192, 8192, 128, True)[0] == 256        # the default's answer for this launch
+    flag_attn.flash_attention(q, q, q, causal=True, dropout_p=0.1)
+    name, args = lib.calls[-1]
+    assert name == "fa_fwd" and args[-2] == 0
+    assert not [w for w in recwarn.list if issubclass(w.category, RuntimeWarning)]
+    monkeypatch.setattr(flash, "get_fwd_config", lambda *a: (256, 64, 5, 4))
+    with pytest.warns(RuntimeWarning, match="without dropout"):
+        flag_attn.flash_attention(q, q, q, causal=True, dropout_p=0.1)
+    assert lib.calls[-1][1][-2] == 128
+    with pytest.warns(RuntimeWarning, match="sm_scale > 0"):
+        flag_attn.flash_attention(q, q, q, causal=True, sm_scale=-1.0)
+    assert lib.calls[-1][1][-2] == 128
+    flag_attn.flash_attention(q, q, q, causal=True)
+    assert lib.calls[-1][1][-2] == 256
+
+
+def test_paged_attention_accepts_any_integer_context_lens_and_keeps_the_query_layout(monkeypatch):
+    """paged.py:16 of the reference returns empty_like(query) and takes context_lens of any integer type."""
+    import flag_attn
+    lib = _with_recording_library(monkeypatch)
+    q = torch.empty(8, 4, 64, dtype=torch.float16).transpose(0, 1)          # (4, 8, 64) view with strides (64, 256, 1)
+    cache = torch.empty(6, 2, 16, 64, dtype=torch.float16)
+    table = torch.zeros(4, 3, dtype=torch.int32)
+    out = flag_attn.paged_attention(q, cache, cache, torch.tensor([3, 40, 0, 17], dtype=torch.int64), table, 0.125, 40)
+    assert out.shape == q.shape and out.stride() == q.stride()
+    name, args = lib.calls[0]
+    assert name == "paged_attn_balanced" and (args[2], args[3]) == (q.stride(0), q.stride(1))
+    with pytest.raises(AssertionError, match="integers"):
+        flag_attn.paged_attention(q, cache, cache, torch.tensor([3., 40., 0., 17.]), table, 0.125, 40)

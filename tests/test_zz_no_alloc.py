@@ -28,6 +28,8 @@ def make_case(seed, num_seqs, Hq, Hkv, D, bs, lo, hi):
 
 def test_static_scratch_entry_point_matches_workspace_entry_point_twice():
     lib = _lib.get()
+    with torch.cuda.device(0):   # what a caller does before it starts a stream capture: resolves the array's address
+        assert lib.paged_attn_balanced_static_prepare() == 0
     num_wgs = 2 * lib.fa_num_cus()
     # first a launch whose pairs are cut over many workgroups, then a smaller one
     for seed, (num_seqs, Hq, Hkv, D, bs, lo, hi) in enumerate([(24, 32, 8, 128, 16, 512, 6000),
