@@ -140,28 +140,57 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, 1) fa_fwd_wide_kernel(FwdParams p) {
       vaddr[db] = lds0 + (uint32_t)(rowl * C::ROW_BYTES + ((4 * (db ^ rho) + 2 * dhalf + ((i & 3) >> 1)) << 4) + (i & 1) * 8);
   }
 
-  // ---- tile loads: wavefront w, instruction j (0..3) fills LDS bytes (4 w + j) * 1024 .. + 1023 of a
-  //      tile = rows 16 w + 4 j + lane / 16, positions lane % 16 ----
-  const int ld_row = 16 * wave + (lane >> 4), ld_pos = lane & 15;   // row of instruction 0
-  uint32_t kchunk_bytes[4];
-#pragma unroll
-  for (int j = 0; j < 4; ++j) kchunk_bytes[j] = (uint32_t)((ld_pos ^ ((ld_row + 4 * j) & 15)) << 4);
-  const uint32_t vchunk_bytes = (uint32_t)((ld_pos ^ (4 * (ld_row & 3))) << 4);   // 4 j does not change row & 3
+  // ---- tile loads: wavefront w, instruction j (0..3) fills LDS bytes j * 4096 + w * 1024 .. + 1023 of a
+  //      tile = rows 16 j + 4 w + lane / 16, positions lane % 16.  A lane's row modulo 16 (what the swizzles
+  //      look at) is the same in all four instructions, so one lane offset serves them and j only moves the
+  //      wave-uniform base ----
+  const int ld_rowl = 4 * wave + (lane >> 4), ld_pos = lane & 15;   // row of instruction j: 16 j + ld_rowl
+  const uint32_t kchunk_bytes = (uint32_t)((ld_pos ^ ld_rowl) << 4);
+  const uint32_t vchunk_bytes = (uint32_t)((ld_pos ^ (4 * (ld_rowl & 3))) << 4);
   const uint32_t kstride_b = (uint32_t)(p.k.st * (int64_t)sizeof(T)), vstride_b = (uint32_t)(p.v.st * (int64_t)sizeof(T));
-  const uint32_t ld_lds = lds0 + (uint32_t)(4 * wave) * 1024u;
+  const uint32_t ld_lds = lds0 + (uint32_t)wave * 1024u;
   // `tile` names the stage; past the last tile the last one is fetched again (into a stage nobody reads
   // any more) so that the loads stay unconditional.  Rows past N re-read row N - 1: their scores are masked.
   auto load_k = [&](int tile, int j) {
     const int n0 = imin(tile, n_tiles - 1) * C::BN;
-    const uint32_t row = (uint32_t)imin(ld_row + 4 * j, N - 1 - n0);
-    hw::dma_load16(kb + (int64_t)n0 * p.k.st, row * kstride_b + kchunk_bytes[j],
-                   ld_lds + (uint32_t)(C::K_BASE + (tile & 1) * C::TILE_BYTES + j * 1024));
+    const uint32_t row = (uint32_t)imin(16 * j + ld_rowl, N - 1 - n0);
+    hw::dma_load16(kb + (int64_t)n0 * p.k.st, row * kstride_b + kchunk_bytes,
+                   ld_lds + (uint32_t)(C::K_BASE + (tile & 1) * C::TILE_BYTES + j * 4096));
   };
   auto load_v = [&](int tile, int j) {
     const int n0 = imin(tile, n_tiles - 1) * C::BN;
-    const uint32_t row = (uint32_t)imin(ld_row + 4 * j, N - 1 - n0);
+    const uint32_t row = (uint32_t)imin(16 * j + ld_rowl, N - 1 - n0);
     hw::dma_load16(vb + (int64_t)n0 * p.v.st, row * vstride_b + vchunk_bytes,
-                   ld_lds + (uint32_t)(C::V_BASE + (tile % 3) * C::TILE_BYTES + j * 1024));
+                   ld_lds + (uint32_t)(C::V_BASE + (tile % 3) * C::TILE_BYTES + j * 4096));
+  };
+  // The same loads for iterations whose tiles (K: i + 3, V: i + 2) exist and are complete, so that nothing needs
+  // clamping: the lane offsets are loop invariants, the wave-uniform source pointers walk on by 16 rows per
+  // instruction (four instructions = one tile = the step to the next iteration) and the LDS stages rotate in
+  // scalar registers.  fast_begin() sets them for iteration i.
+  const uint32_t koff_fast = (uint32_t)ld_rowl * kstride_b + kchunk_bytes, voff_fast = (uint32_t)ld_rowl * vstride_b + vchunk_bytes;
+  const char* ksrc_fast = nullptr;
+  const char* vsrc_fast = nullptr;
+  uint32_t kdst_fast = 0, vdst_fast = 0;
+  auto fast_begin = [&](int i) {
+    ksrc_fast = (const char*)(kb + (int64_t)(i + 3) * C::BN * p.k.st);
+    vsrc_fast = (const char*)(vb + (int64_t)(i + 2) * C::BN * p.v.st);
+    kdst_fast = ld_lds + (uint32_t)(C::K_BASE + ((i + 3) & 1) * C::TILE_BYTES);
+    vdst_fast = ld_lds + (uint32_t)(C::V_BASE + ((i + 2) % 3) * C::TILE_BYTES);
+  };
+  auto load_k_fast = [&](auto j_tag) {
+    constexpr int j = decltype(j_tag)::value;
+    hw::dma_load16_at<j * 4096>(ksrc_fast, koff_fast, kdst_fast);
+    ksrc_fast += 16 * (int64_t)kstride_b;
+    if constexpr (j == 3) kdst_fast ^= (uint32_t)C::TILE_BYTES;   // the two K stages differ in this address bit alone (the LDS allocation starts at a multiple of 2 TILE_BYTES)
+  };
+  auto load_v_fast = [&](auto j_tag) {
+    constexpr int j = decltype(j_tag)::value;
+    hw::dma_load16_at<j * 4096>(vsrc_fast, voff_fast, vdst_fast);
+    vsrc_fast += 16 * (int64_t)vstride_b;
+    if constexpr (j == 3) {
+      const uint32_t last = ld_lds + (uint32_t)(C::V_BASE + 2 * C::TILE_BYTES);
+      vdst_fast = vdst_fast == last ? vdst_fast - 2 * (uint32_t)C::TILE_BYTES : vdst_fast + (uint32_t)C::TILE_BYTES;
+    }
   };
 
   // ---- state ----
@@ -173,17 +202,25 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, 1) fa_fwd_wide_kernel(FwdParams p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) S[x][h][r] = 0.f;
   u32x4 P[2][4];       // [block][group]: probabilities rounded to T, the B operand of the second product
-  f32x16 O[2][4];      // [block][32-wide slice of D]: O^T, in AGPRs
-  static_for<8>([&](auto i) { hw::pinned_o_clear<decltype(i)::value>(O[decltype(i)::value / 4][decltype(i)::value % 4]); });
+  // [block][32-wide slice of D]: O^T.  On the GPU it lives in a[0:127], which only the pinned_o_* statements
+  // name (they hide those registers from the compiler, see pinned_regs.hpp); this array carries the values in the
+  // host simulator build and is never touched on the GPU.
+  hw::o_tuples O;
   const float c2 = p.sm_scale * kLog2e;
   const float tau = C::kTau / c2;           // in units of raw scores (sm_scale > 0)
-  float m_ref[2] = {neg_inf(), neg_inf()};  // reference maximum of the exponentials (raw score units)
-  float shift[2] = {0.f, 0.f};              // -m_ref * c2 (0 while no key has been seen)
+  // Reference maximum of the exponentials (raw score units).  A row that has seen no key yet holds a large
+  // finite stand-in instead of -inf, so that -m_ref * c2 and differences of references need no special cases:
+  // exp2(c2 (-inf - m_ref)) is 0 for a masked score and exp2(c2 (m_ref - m_new)) is 0 when the first key arrives.
+  constexpr float kNoKeyYet = -1e30f;
+  float m_ref[2] = {kNoKeyYet, kNoKeyYet};
+  float shift[2] = {0.f, 0.f};              // -m_ref * c2 (set by a half's decision before its first multiply-add)
   float lsum[2][2] = {{0.f, 0.f}, {0.f, 0.f}};   // [block][partial]: this lane's part of the row sum (fp32, before rounding)
   // decisions of the two halves of a tile: factor by which O and the row sums move to the new reference
-  float alpha[2][2] = {{1.f, 1.f}, {1.f, 1.f}};   // [half][block]
+  // decisions of the two halves of a tile: by how much the reference moved (old - new, 0 where it stays); O and
+  // the row sums are multiplied by exp2(c2 * moved) in the rare wavefront-uniform branch between two runs
+  float moved[2][2] = {{0.f, 0.f}, {0.f, 0.f}};   // [half][block]
   bool changed[2] = {false, false};               // [half]
-  float m_new[2] = {neg_inf(), neg_inf()}, shift_new[2] = {0.f, 0.f};
+  float m_new[2] = {kNoKeyYet, kNoKeyYet}, shift_new[2] = {0.f, 0.f};
   float mx[2] = {neg_inf(), neg_inf()};
   float xpend = 0.f;    // multiply-add result waiting for its exponential
   float ering[6] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};   // exponentials waiting to be summed and packed
@@ -208,9 +245,10 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, 1) fa_fwd_wide_kernel(FwdParams p) {
   // of tile i + 1 (if DO_S), the last 16 add the same keys of tile i to O (if DO_PV).  The vector work
   // belongs to tile i (steps 34.. of its exponential pass, if DO_PV) and to tile i + 1 (row maxima and
   // steps ..33, if DO_S).  MASKED: tile i + 1 needs the key tail / causal select.
-  auto half_iteration = [&](auto half_tag, auto masked_tag, auto do_s_tag, auto do_pv_tag, int i) {
+  auto half_iteration = [&](auto half_tag, auto masked_tag, auto do_s_tag, auto do_pv_tag, auto fast_tag, int i) {
     constexpr int HALF = decltype(half_tag)::value;
     constexpr bool MASKED = decltype(masked_tag)::value, DO_S = decltype(do_s_tag)::value, DO_PV = decltype(do_pv_tag)::value;
+    constexpr bool FAST = decltype(fast_tag)::value;   // the tiles this iteration fetches need no clamping (load_k_fast)
     if constexpr (MASKED && DO_S && HALF == 0) {
       const int n0 = (i + 1) * C::BN;
 #pragma unroll
@@ -226,27 +264,18 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, 1) fa_fwd_wide_kernel(FwdParams p) {
       if constexpr (kl < 16) {
         if constexpr (DO_S) {
           constexpr int q = k / 2, x = k % 2, kk = q % 8;
-          if constexpr (kk == 0) hw::pinned_s_mfma_first<2 * x + HALF>(ring[q % 4], qreg[x][kk], S[x][HALF]);
-          else hw::pinned_s_mfma<2 * x + HALF>(ring[q % 4], qreg[x][kk], S[x][HALF]);
+          if constexpr (kk == 0) hw::pinned_s_mfma_first<2 * x + HALF>(ring[q % 4], qreg[x][kk], S[x][HALF], O);
+          else hw::pinned_s_mfma<2 * x + HALF>(ring[q % 4], qreg[x][kk], S[x][HALF], O);
         }
       } else {
         if constexpr (DO_PV) {
           constexpr int q = k / 2, x = k % 2, g = 2 * HALF + (q % 8) / 4, db = q % 4;
-          hw::pinned_o_mfma<4 * x + db>(ring[q % 4], hw::as_v8<T>(P[x][g]), O[x][db]);
+          hw::pinned_o_mfma<4 * x + db>(ring[q % 4], hw::as_v8<T>(P[x][g]), O);
         }
       }
       // Iteration -1 has no second product: the slots behind its S run hold no matrix instruction, and the
       // vector work of slot kMax would follow the run's last products too closely (hazard distances above)
       if constexpr (DO_S && !DO_PV && kl == 16) hw::mfma_drain();
-      // ------------------------------------------------- operand of the slot pair kLead ahead
-      if constexpr (k % 2 == 0) {
-        constexpr int q = (k + C::kLead) / 2;
-        if constexpr (q < 32) {
-          if constexpr ((q % 16 < 8 && DO_S) || (q % 16 >= 8 && DO_PV)) request(std::integral_constant<int, q>{});
-        } else {   // operands 0..2 of the next iteration: kaddr already points at the other K stage
-          request(std::integral_constant<int, q - 32>{});
-        }
-      }
       // ---------------------------------------------------------------- stages, barrier, tile loads
       // all K operands of this iteration have been requested by slot 40 (operand 23): toggle the K stage
       if constexpr (k >= 41 && k < 41 + C::KSTEPS / 2) {
@@ -262,33 +291,40 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, 1) fa_fwd_wide_kernel(FwdParams p) {
       }
       if constexpr (k == C::kBarrierSlot - 1) hw::wait_global_loads();
       if constexpr (k == C::kBarrierSlot) hw::barrier_only();
-      if constexpr (k >= C::kLoadSlot && k < C::kLoadSlot + 4) load_k(i + 3, k - C::kLoadSlot);
-      if constexpr (k >= C::kLoadSlot + 4 && k < C::kLoadSlot + 8) load_v(i + 2, k - C::kLoadSlot - 4);
+      if constexpr (k >= C::kLoadSlot && k < C::kLoadSlot + 4) {
+        if constexpr (FAST) load_k_fast(std::integral_constant<int, k - C::kLoadSlot>{});
+        else load_k(i + 3, k - C::kLoadSlot);
+      }
+      if constexpr (k >= C::kLoadSlot + 4 && k < C::kLoadSlot + 8) {
+        if constexpr (FAST) load_v_fast(std::integral_constant<int, k - C::kLoadSlot - 4>{});
+        else load_v(i + 2, k - C::kLoadSlot - 4);
+      }
       // ---------------------------------------------------------------- row maximum of this half of tile i + 1
       if constexpr (DO_S) {
         if constexpr (kl >= C::kMax && kl < C::kMax + 8) {
-          static_for<2>([&](auto u) {
-            constexpr int j = (kl - C::kMax) * 2 + decltype(u)::value, x = j / 8, r0 = 2 * (j % 8);
+          static_for<2>([&](auto u) {   // one step of each block per slot: consecutive instructions are independent
+            constexpr int x = decltype(u)::value, r0 = 2 * (kl - C::kMax);
             f32x16& s = S[x][HALF];
             if constexpr (MASKED) {   // key 32 HALF + 8 (r / 4) + r % 4 + 4 hh of the tile is visible iff <= lim
               s[r0] = (HALF * 32 + 8 * (r0 / 4) + r0 % 4 <= rel[x]) ? s[r0] : neg_inf();
               s[r0 + 1] = (HALF * 32 + 8 * ((r0 + 1) / 4) + (r0 + 1) % 4 <= rel[x]) ? s[r0 + 1] : neg_inf();
             }
-            if constexpr (r0 == 0) mx[x] = hw::max2(s[0], s[1]);
-            else mx[x] = hw::max3(mx[x], s[r0], s[r0 + 1]);
-            hw::pin(mx[x]);
+            if constexpr (r0 == 0) mx[x] = hw::slot_max2(s[0], s[1]);
+            else mx[x] = hw::slot_max3(mx[x], s[r0], s[r0 + 1]);
           });
         }
         // a row lives in lanes l and l ^ 32: [A.lo, B.lo] vs [A.hi, B.hi], then both halves get both
-        if constexpr (kl == C::kSwap) hw::swap_halves(mx[0], mx[1]);
+        // (with a second product in the slots, the exchange sits at the end of its slot, below: the slot's own
+        // vector work then supplies the wait states the exchange needs before it, the next slot's matrix
+        // instruction those behind it)
+        if constexpr (!DO_PV && (kl == C::kSwap || kl == C::kSwap + 2)) hw::swap_halves(mx[0], mx[1]);
         if constexpr (kl == C::kSwap + 1) { mx[0] = hw::max2(mx[0], mx[1]); mx[1] = mx[0]; }
-        if constexpr (kl == C::kSwap + 2) hw::swap_halves(mx[0], mx[1]);
         if constexpr (kl == C::kFinal || kl == C::kFinal + 1) {
           constexpr int x = kl - C::kFinal;
           const bool grow = mx[x] > m_ref[x] + tau;   // always on the first half with a visible key
           m_new[x] = grow ? mx[x] : m_ref[x];
-          alpha[HALF][x] = grow ? hw::exp2_fast((m_ref[x] - m_new[x]) * c2) : 1.f;
-          shift_new[x] = (m_new[x] == neg_inf()) ? 0.f : -m_new[x] * c2;
+          moved[HALF][x] = m_ref[x] - m_new[x];
+          shift_new[x] = -m_new[x] * c2;
           if constexpr (x == 0) changed[HALF] = grow;
           else changed[HALF] = changed[HALF] || grow;
         }
@@ -297,6 +333,9 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, 1) fa_fwd_wide_kernel(FwdParams p) {
           for (int x = 0; x < 2; ++x) { m_ref[x] = m_new[x]; shift[x] = shift_new[x]; }
         }
       }
+      // the last iteration decides nothing: what its predecessor decided for this half has been applied to O
+      // before this run, and must not reach the row sums a second time at the next boundary
+      if constexpr (!DO_S && kl == C::kFinal) { moved[HALF][0] = 0.f; moved[HALF][1] = 0.f; changed[HALF] = false; }
       // ---------------------------------------------------------------- exponential passes
       // Step t of a tile's exponential pass: the multiply-add of element t, the exponential of element
       // t - 1, the row-sum update with element t - 2 and, every other step, the pack of elements t - 4 and
@@ -305,36 +344,38 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, 1) fa_fwd_wide_kernel(FwdParams p) {
         constexpr int t = decltype(t_tag)::value;
         if constexpr (t >= 4 && t <= 66 && t % 2 == 0) {
           constexpr ExpStep e(t - 3);
-          uint32_t w = hw::pack2(T{}, ering[(t - 4) % 6], ering[(t - 3) % 6]);
-          hw::pin(w);
-          P[e.x][e.g][e.word] = w;
+          P[e.x][e.g][e.word] = hw::slot_pack2(T{}, ering[(t - 4) % 6], ering[(t - 3) % 6]);
         }
         if constexpr (t >= 2 && t <= 65) {   // two partial sums per block, so that consecutive updates are independent
           constexpr ExpStep e(t - 2);
-          lsum[e.x][(e.r / 2) % 2] += ering[(t - 2) % 6];
-          hw::pin(lsum[e.x][(e.r / 2) % 2]);
+          hw::slot_add(lsum[e.x][(e.r / 2) % 2], ering[(t - 2) % 6]);
         }
-        if constexpr (t >= 1 && t <= 64) { ering[(t - 1) % 6] = hw::exp2_fast(xpend); hw::pin(ering[(t - 1) % 6]); }
+        if constexpr (t >= 1 && t <= 64) ering[(t - 1) % 6] = hw::slot_exp2(xpend);
         if constexpr (t <= 63) {
           constexpr ExpStep e(t);
-          xpend = fmaf(S[e.x][e.kb][e.r], c2, shift[e.x]);
-          hw::pin(xpend);
+          xpend = hw::slot_fma(S[e.x][e.kb][e.r], c2, shift[e.x]);
         }
       };
-      // the row sums move to a half's reference between the last update of the half before it (steps 33 / 65,
-      // slots 63 / 31) and its own first update (steps 34 / 2, slots 0 / 32)
-      if constexpr (DO_PV && k == 0) {
-#pragma unroll
-        for (int x = 0; x < 2; ++x) { lsum[x][0] *= alpha[1][x]; lsum[x][1] *= alpha[1][x]; }
-      }
-      if constexpr (DO_S && k == C::kExp0 + 2) {
-#pragma unroll
-        for (int x = 0; x < 2; ++x) { lsum[x][0] *= alpha[0][x]; lsum[x][1] *= alpha[0][x]; }
-      }
+      // (the row sums move to a half's reference between the last update of the half before it -- steps 33 / 65,
+      // slots 63 / 31 -- and its own first update -- steps 34 / 2, slots 0 / 32: at the boundary between two runs,
+      // in rescale() below)
       // tile i: steps 34 + k (slots 30 to 32 only finish its last elements); placed before tile i + 1's step
       // of the same slot, because step 64 reads the pending multiply-add that step 0 overwrites
       if constexpr (DO_PV && k < C::kExp0 + 3) exp_step(std::integral_constant<int, k + 64 - C::kExp0>{});
       if constexpr (DO_S && k >= C::kExp0) exp_step(std::integral_constant<int, k - C::kExp0>{});
+      if constexpr (DO_S && DO_PV && (kl == C::kSwap || kl == C::kSwap + 2)) hw::swap_halves_in_slot(mx[0], mx[1]);
+      // ------------------------------------------------- operand of the slot pair kLead ahead
+      // (last in its slot: the compiler pads two assembly statements that touch the same register and have no
+      // instruction it knows between them with an s_nop; the LDS read of an even slot and the wait for an
+      // operand before an odd slot's successor put one at every slot boundary)
+      if constexpr (k % 2 == 0) {
+        constexpr int q = (k + C::kLead) / 2;
+        if constexpr (q < 32) {
+          if constexpr ((q % 16 < 8 && DO_S) || (q % 16 >= 8 && DO_PV)) request(std::integral_constant<int, q>{});
+        } else {   // operands 0..2 of the next iteration: kaddr already points at the other K stage
+          request(std::integral_constant<int, q - 32>{});
+        }
+      }
       hw::sched_fence();
     });
   };
@@ -362,15 +403,26 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, 1) fa_fwd_wide_kernel(FwdParams p) {
     using H1 = std::integral_constant<int, 1>;
     using Yes = std::true_type;
     using No = std::false_type;
-    // O moves to a half's reference right before the products of that half's probabilities
+    // Between two runs: O moves to the reference of the half whose probabilities the coming run multiplies
+    // (decided one iteration ago), and the row sums to the reference of the half whose exponentials the coming
+    // run starts to add (decided in the run just finished: it is the other half).  Either happens only when some
+    // row's reference moved, which is rare: one wavefront-uniform branch covers both.
     auto rescale = [&](auto half_tag) {
       constexpr int h = decltype(half_tag)::value;
-      if (hw::wave_any(changed[h])) {
+      if (hw::wave_any(changed[0] || changed[1])) {
         hw::keep_branch();
         hw::mfma_drain();
+        float to_o[2], to_sum[2];
+#pragma unroll
+        for (int x = 0; x < 2; ++x) {
+          to_o[x] = hw::exp2_fast(moved[h][x] * c2);
+          to_sum[x] = hw::exp2_fast(moved[1 - h][x] * c2);
+          lsum[x][0] *= to_sum[x];
+          lsum[x][1] *= to_sum[x];
+        }
         static_for<8>([&](auto i) {
           constexpr int x = decltype(i)::value / 4, db = decltype(i)::value % 4;
-          hw::pinned_o_scale<4 * x + db>(O[x][db], alpha[h][x]);
+          hw::pinned_o_scale<4 * x + db>(O, to_o[x]);
         });
         hw::mfma_drain();   // the rewritten accumulators are read by matrix instructions next
       }
@@ -380,29 +432,49 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, 1) fa_fwd_wide_kernel(FwdParams p) {
     // one loop the register allocator gives up on keeping S, O and Q in place.  Masked tiles come last (the
     // key tail, and under the causal mask the tiles on and above the wavefront's diagonal).
     // iteration -1: S(0) only.  Its V stage advance (to tile 0's stage) is the identity.
-    if (tile_masked(0)) { half_iteration(H0{}, Yes{}, Yes{}, No{}, -1); half_iteration(H1{}, Yes{}, Yes{}, No{}, -1); }
-    else { half_iteration(H0{}, No{}, Yes{}, No{}, -1); half_iteration(H1{}, No{}, Yes{}, No{}, -1); }
+    // (cleared here, next to the first statements that hide a[0:127] from the compiler: earlier, the prologue's
+    // own code could still use those registers)
+    static_for<8>([&](auto t) { hw::pinned_o_clear<decltype(t)::value>(O); });
+    if (tile_masked(0)) { half_iteration(H0{}, Yes{}, Yes{}, No{}, No{}, -1); half_iteration(H1{}, Yes{}, Yes{}, No{}, No{}, -1); }
+    else { half_iteration(H0{}, No{}, Yes{}, No{}, No{}, -1); half_iteration(H1{}, No{}, Yes{}, No{}, No{}, -1); }
     int i = 0;
+    // tiles [0, n_plain) are crossed by no mask for this wavefront: complete, and under the causal mask wholly
+    // visible to its first row (tile t: 64 t + 63 <= mw + pseq)
+    int n_plain = N / C::BN;
+    if (p.causal) n_plain = imin(n_plain, imax(0, mw + pseq + 1) / C::BN);
+    const int end_plain = imin(n_tiles, n_plain) - 1;                   // iterations i < end_plain form S of a plain tile i + 1
+    // of these, the ones whose fetched tiles (up to tile i + 3) exist and are complete
+    const int end_fast = imin(end_plain, imin(n_tiles, N / C::BN) - 3);
+    fast_begin(0);
 #pragma unroll 1
-    for (; i + 1 < n_tiles && !tile_masked(i + 1); ++i) {
+    for (; i < end_fast; ++i) {
       rescale(H0{});
-      half_iteration(H0{}, No{}, Yes{}, Yes{}, i);
+      half_iteration(H0{}, No{}, Yes{}, Yes{}, Yes{}, i);
       rescale(H1{});
-      half_iteration(H1{}, No{}, Yes{}, Yes{}, i);
+      half_iteration(H1{}, No{}, Yes{}, Yes{}, Yes{}, i);
+    }
+#pragma unroll 1
+    for (; i < end_plain; ++i) {
+      rescale(H0{});
+      half_iteration(H0{}, No{}, Yes{}, Yes{}, No{}, i);
+      rescale(H1{});
+      half_iteration(H1{}, No{}, Yes{}, Yes{}, No{}, i);
     }
 #pragma unroll 1
     for (; i + 1 < n_tiles; ++i) {
       rescale(H0{});
-      half_iteration(H0{}, Yes{}, Yes{}, Yes{}, i);
+      half_iteration(H0{}, Yes{}, Yes{}, Yes{}, No{}, i);
       rescale(H1{});
-      half_iteration(H1{}, Yes{}, Yes{}, Yes{}, i);
+      half_iteration(H1{}, Yes{}, Yes{}, Yes{}, No{}, i);
     }
     rescale(H0{});
-    half_iteration(H0{}, No{}, No{}, Yes{}, i);
+    half_iteration(H0{}, No{}, No{}, Yes{}, No{}, i);
     rescale(H1{});
-    half_iteration(H1{}, No{}, No{}, Yes{}, i);
+    half_iteration(H1{}, No{}, No{}, Yes{}, No{}, i);
     hw::wait_global_loads();   // the unconditional loads of the last iterations must not outlive the LDS allocation
     hw::mfma_drain();
+  } else {   // no key is visible to any row of the workgroup: the epilogue writes zeros
+    static_for<8>([&](auto t) { hw::pinned_o_clear<decltype(t)::value>(O); });
   }
 
   // ---- epilogue: O = acc / l, L = m * scale + ln(l); rows that saw no key give O = 0, L = -inf ----
@@ -418,8 +490,8 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, 1) fa_fwd_wide_kernel(FwdParams p) {
         constexpr int db = decltype(j_tag)::value / 4, g = decltype(j_tag)::value % 4, I = 4 * x + db;
         const int d = db * 32 + 8 * g + 4 * hh;
         hw::u32x2 w;
-        w[0] = hw::pack2(T{}, hw::pinned_o_read<I, 4 * g + 0>(O[x][db]) * inv, hw::pinned_o_read<I, 4 * g + 1>(O[x][db]) * inv);
-        w[1] = hw::pack2(T{}, hw::pinned_o_read<I, 4 * g + 2>(O[x][db]) * inv, hw::pinned_o_read<I, 4 * g + 3>(O[x][db]) * inv);
+        w[0] = hw::pack2(T{}, hw::pinned_o_read<I, 4 * g + 0>(O) * inv, hw::pinned_o_read<I, 4 * g + 1>(O) * inv);
+        w[1] = hw::pack2(T{}, hw::pinned_o_read<I, 4 * g + 2>(O) * inv, hw::pinned_o_read<I, 4 * g + 3>(O) * inv);
         *(hw::u32x2*)(ob + d) = w;
       });
       if (hh == 0)

@@ -144,6 +144,10 @@ FA_DEVICE void swap_halves(float& a, float& b) {
   asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
 }
 
+// The exchange alone, for hand-placed streams: the CALLER keeps two instructions that do not touch a or b on
+// either side of it.
+FA_DEVICE void swap_halves_in_slot(float& a, float& b) { asm volatile("v_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b)); }
+
 // Tells the compiler that x has the same value in every lane (kept in a scalar register).
 FA_DEVICE int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
 
@@ -160,6 +164,13 @@ FA_DEVICE u32x4 load_streaming(const void* p) { return __builtin_nontemporal_loa
 FA_DEVICE void dma_load16(const void* base, uint32_t lane_offset, uint32_t lds_base) {
   // (one wait state between the scalar write of M0 and the instruction that reads it)
   asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(lane_offset), "s"(base), "s"(lds_base) : "memory", "m0");
+}
+// The same with a compile-time addition to the LDS base (a fixed place inside a rotating stage): the sum goes
+// straight into M0, one scalar instruction.
+template <int LDS_OFFSET>
+FA_DEVICE void dma_load16_at(const void* base, uint32_t lane_offset, uint32_t lds_base) {
+  asm volatile("s_add_u32 m0, %2, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               : : "v"(lane_offset), "s"(base), "s"(lds_base), "n"(LDS_OFFSET) : "memory", "m0", "scc");
 }
 // LDS byte address of a pointer into the workgroup's LDS allocation.
 FA_DEVICE uint32_t lds_address(const void* p) {
@@ -200,6 +211,50 @@ FA_DEVICE void sched_prefetched_operands() {
 
 FA_DEVICE float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
 FA_DEVICE float log_nat(float x) { return __logf(x); }
+
+// Vector-ALU steps that stay exactly where the source puts them ("slotted" variants for the hand-placed
+// instruction streams).  The scheduling fence binds the instruction scheduler only: earlier passes move
+// side-effect-free arithmetic across it, towards its operands or its first use, and so fill one slot with the
+// work of two and leave the next one empty.  A wavefront that is alone on its SIMD issues one instruction per
+// 4 clocks whatever its kind (8 for an exponential), so what a slot holds beyond about five instructions is not
+// hidden under its matrix instruction; these keep a slot's share in that slot.  The compiler does not see into
+// them: the CALLER keeps one other instruction between an exponential and the first use of its result.
+FA_DEVICE float slot_fma(float a, float b, float c) {
+  float r;
+  asm volatile("v_fma_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+FA_DEVICE float slot_mul(float a, float b) {
+  float r;
+  asm volatile("v_mul_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+FA_DEVICE float slot_exp2(float x) {
+  float r;
+  asm volatile("v_exp_f32 %0, %1" : "=v"(r) : "v"(x));
+  return r;
+}
+FA_DEVICE float slot_max3(float a, float b, float c) {
+  float r;
+  asm volatile("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+FA_DEVICE float slot_max2(float a, float b) {
+  float r;
+  asm volatile("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+FA_DEVICE void slot_add(float& acc, float x) { asm volatile("v_add_f32 %0, %0, %1" : "+v"(acc) : "v"(x)); }
+FA_DEVICE uint32_t slot_pack2(half_t, float a, float b) {
+  uint32_t r;
+  asm volatile("v_cvt_pk_f16_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+FA_DEVICE uint32_t slot_pack2(bf16_t, float a, float b) {
+  uint32_t r;
+  asm volatile("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
 
 // Two fp32 values rounded to T and packed (lo = a, hi = b), and acc + lo + hi of such a pair.
 FA_DEVICE uint32_t pack2(half_t, float a, float b) {

@@ -266,12 +266,13 @@ inline f32x16 mfma32(half8 a, half8 b, f32x16 c) { return mfma32_any(a, b, c); }
 inline f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) { return mfma32_any(a, b, c); }
 inline f32x16 zero16() { f32x16 z; for (int r = 0; r < 16; ++r) z[r] = 0.f; return z; }
 // accumulator tuples that the GPU build pins to fixed physical registers: plain values here
-template <int I, class V8> inline void pinned_o_mfma(V8 a, V8 b, f32x16& c) { c = mfma32_any(a, b, c); }
-template <int I, class V8> inline void pinned_s_mfma_first(V8 a, V8 b, f32x16& c) { c = mfma32_any(a, b, zero16()); }
-template <int I, class V8> inline void pinned_s_mfma(V8 a, V8 b, f32x16& c) { c = mfma32_any(a, b, c); }
-template <int I> inline void pinned_o_clear(f32x16& c) { c = zero16(); }
-template <int I> inline void pinned_o_scale(f32x16& c, float f) { for (int r = 0; r < 16; ++r) c[r] *= f; }
-template <int I, int R> inline float pinned_o_read(const f32x16& c) { return c[R]; }
+using o_tuples = f32x16[2][4];
+template <int I, class V8> inline void pinned_o_mfma(V8 a, V8 b, o_tuples& o) { o[I / 4][I % 4] = mfma32_any(a, b, o[I / 4][I % 4]); }
+template <int I, class V8> inline void pinned_s_mfma_first(V8 a, V8 b, f32x16& c, o_tuples&) { c = mfma32_any(a, b, zero16()); }
+template <int I, class V8> inline void pinned_s_mfma(V8 a, V8 b, f32x16& c, o_tuples&) { c = mfma32_any(a, b, c); }
+template <int I> inline void pinned_o_clear(o_tuples& o) { o[I / 4][I % 4] = zero16(); }
+template <int I> inline void pinned_o_scale(o_tuples& o, float f) { for (int r = 0; r < 16; ++r) o[I / 4][I % 4][r] *= f; }
+template <int I, int R> inline float pinned_o_read(const o_tuples& o) { return o[I / 4][I % 4][R]; }
 inline void mfma_drain() {}
 inline f32x16 mfma32_vacc(half8 a, half8 b, f32x16 c) { return mfma32_any(a, b, c); }
 inline f32x16 mfma32_vacc(bf16x8 a, bf16x8 b, f32x16 c) { return mfma32_any(a, b, c); }
@@ -349,11 +350,15 @@ inline void swap_halves(float& a, float& b) {
   a = na;
   b = nb;
 }
+inline void swap_halves_in_slot(float& a, float& b) { swap_halves(a, b); }
 inline float max3(float a, float b, float c) { return fmaxf(fmaxf(a, b), c); }
 inline float max2(float a, float b) { return fmaxf(a, b); }
 inline uint32_t lds_address(const void* p) { return (uint32_t)((const unsigned char*)p - hwsim::lds); }
 inline void dma_load16(const void* base, uint32_t lane_offset, uint32_t lds_base) {
   memcpy(hwsim::lds + lds_base + 16 * (hwsim::cur & 63), (const char*)base + lane_offset, 16);
+}
+template <int LDS_OFFSET> inline void dma_load16_at(const void* base, uint32_t lane_offset, uint32_t lds_base) {
+  dma_load16(base, lane_offset, lds_base + LDS_OFFSET);
 }
 inline uint32_t pack2(half_t, float a, float b) {
   half_t v[2] = {(half_t)a, (half_t)b};
@@ -377,5 +382,13 @@ inline void keep_branch() {}
 template <int N, int DEPTH, int RPM = 1, int EXTRA = 0> inline void sched_prefetched_operands() {}
 inline float exp2_fast(float x) { return exp2f(x); }
 inline float log_nat(float x) { return logf(x); }
+inline float slot_fma(float a, float b, float c) { return fmaf(a, b, c); }
+inline float slot_mul(float a, float b) { return a * b; }
+inline float slot_exp2(float x) { return exp2f(x); }
+inline float slot_max3(float a, float b, float c) { return fmaxf(fmaxf(a, b), c); }
+inline float slot_max2(float a, float b) { return fmaxf(a, b); }
+inline void slot_add(float& acc, float x) { acc += x; }
+inline uint32_t slot_pack2(half_t t, float a, float b) { return pack2(t, a, b); }
+inline uint32_t slot_pack2(bf16_t t, float a, float b) { return pack2(t, a, b); }
 
 }  // namespace hw

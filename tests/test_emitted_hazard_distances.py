@@ -304,3 +304,71 @@ def test_the_needed_distance_is_the_one_the_compiler_pads_to(obj, tmp_path):
     where it had nothing else to put in between, the distance it left is the requirement."""
     results = _audit(obj, tmp_path)
     assert min(worst["read"][0] for worst, _ in results.values()) == 0
+
+
+def _wait_states(ins):
+    return int(ins.split()[1]) + 1 if ins.startswith("s_nop") else 1
+
+
+def slotted_vector_hazards(lines):
+    """What the hand-placed vector instructions of the 256-row forward have to keep by themselves, because they are
+    inline assembly: (a) the output tuples a[0:127] are written by matrix instructions, by the clearing writes of 0
+    and by the read-scale-write triple only -- never by a copy of the compiler's; (b) the result of an exponential
+    is not read by the very next instruction; (c) two wait states separate a lane exchange from the instructions
+    that write or read its registers.  Returns a list of complaints; checks run inside basic blocks."""
+    body = [l for l in lines if l and not l.endswith(":")]
+    bad = []
+    for i, ins in enumerate(body):
+        op, _, rest = ins.partition(" ")
+        operands = [o.strip() for o in rest.split(",")]
+        if op == "v_accvgpr_write_b32":
+            dst = next(iter(_vgprs(operands[0])))
+            if dst[0] == "a" and dst[1] < 128 and operands[1] != "0":
+                triple = body[i - 3] if i >= 3 else ""
+                if triple != f"v_accvgpr_read_b32 {operands[1]}, {operands[0]}":
+                    bad.append(f"(a) {ins}: a write to the output tuples that is not the scaling triple")
+        elif op.startswith("v_exp_f32") and i + 1 < len(body):
+            nxt = body[i + 1]
+            if not nxt.startswith(("s_", "v_mfma")) and _vgprs(operands[0]) & _vgprs(nxt.partition(" ")[2].partition(",")[2]):
+                bad.append(f"(b) {nxt} reads the exponential of the instruction before it")
+        elif op == "v_permlane32_swap_b32":
+            regs = _vgprs(rest)
+            for step, seq in ((-1, body[:i][::-1]), (1, body[i + 1:])):
+                states = 0
+                for other in seq:
+                    if states >= 2 or other.startswith(("s_branch", "s_cbranch", "s_endpgm")):
+                        break
+                    if not other.startswith("s_") and _vgprs(other.partition(" ")[2]) & regs:
+                        bad.append(f"(c) {other} is {states} wait states {'before' if step < 0 else 'behind'} {ins}")
+                    states += _wait_states(other)
+    return bad
+
+
+def test_the_slotted_vector_audit_sees_each_kind_of_mistake():
+    ok = ["v_accvgpr_write_b32 a5, 0", "v_accvgpr_read_b32 v9, a17", "v_mul_f32_e32 v9, v9, v3", "s_nop 0",
+          "v_accvgpr_write_b32 a17, v9", "v_accvgpr_write_b32 a130, v4", "v_exp_f32_e32 v7, v8", "v_add_f32_e32 v1, v1, v2",
+          "v_add_f32_e32 v1, v1, v7", "v_mov_b32_e32 v20, v1", "s_nop 1", "v_permlane32_swap_b32_e32 v20, v21", "s_nop 0",
+          "v_mfma_f32_32x32x16_bf16 a[0:15], v[2:5], v[6:9], a[0:15]", "v_max_f32_e32 v20, v20, v21"]
+    ok = [l.replace("v_permlane32_swap_b32_e32", "v_permlane32_swap_b32") for l in ok]
+    assert slotted_vector_hazards(ok) == []
+    assert len(slotted_vector_hazards(["v_accvgpr_write_b32 a16, v169"])) == 1
+    assert len(slotted_vector_hazards(["v_exp_f32_e32 v7, v8", "v_add_f32_e32 v1, v1, v7"])) == 1
+    assert len(slotted_vector_hazards(["v_mov_b32_e32 v20, v1", "s_nop 0", "v_permlane32_swap_b32 v20, v21"])) == 1
+    assert len(slotted_vector_hazards(["v_permlane32_swap_b32 v20, v21", "v_mfma_f32_32x32x16_bf16 a[0:15], v[2:5], v[6:9], a[0:15]",
+                                       "v_max_f32_e32 v20, v20, v21"])) == 1
+
+
+def test_hand_placed_vector_instructions_of_the_256_row_forward_keep_their_distances(tmp_path):
+    path = os.path.join(BUILD, "fa_fwd_wide.o")
+    if not os.path.exists(path) or not all(shutil.which(os.path.join(LLVM, t)) for t in
+                                           ("llvm-objcopy", "clang-offload-bundler", "llvm-objdump")):
+        pytest.skip("needs the objects of a library build and the LLVM binary tools")
+    audited = 0
+    for name, lines in _disassemble(path, tmp_path).items():
+        if "fa_fwd_wide_kernel" in name:
+            audited += 1
+            lines = [re.sub(r"\bv_permlane32_swap_b32_e32\b", "v_permlane32_swap_b32", l) for l in lines]
+            assert slotted_vector_hazards(lines) == [], name
+            assert sum(l.startswith("v_permlane32_swap") for l in lines) >= 8
+            assert sum(l.startswith("v_accvgpr_write_b32") for l in lines) >= 256
+    assert audited == 2
