@@ -94,17 +94,23 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, 1) fa_fwd_wide_kernel(FwdParams p) {
 
   const int tid = hw::thread_id(), lane = tid & 63, wave = hw::uniform(tid >> 6);
   const int l32 = lane & 31, hh = lane >> 5;
-  const TileId wg = tile_of_workgroup(p.H, p.B);
+  // With the key axis in pieces a workgroup owns (row block, head, piece); the piece index runs fastest, so the
+  // pieces of a head share an XCD's L2 with its other row blocks.
+  const int pieces = p.num_splits > 0 ? p.num_splits : 1;
+  const TileId wg = tile_of_workgroup(p.H * pieces, p.B);
   const int mb = (p.M + C::BM - 1) / C::BM - 1 - wg.rank;  // long rows first under the causal mask
-  const int head = wg.head, batch = wg.batch;
+  const int head = wg.head / pieces, piece = wg.head - head * pieces, batch = wg.batch;
   const int hk = head / p.group;
-  const int M = p.M, N = p.N, pseq = N - M;
+  // keys first_key .. first_key + N - 1 of the p.N keys; everything below works on the piece as if it were the
+  // whole key axis: key index relative to first_key, pseq the offset of the causal diagonal in those terms
+  const int first_key = piece * (p.num_splits > 0 ? p.split_size : 0);
+  const int M = p.M, N = imin(p.N - first_key, p.num_splits > 0 ? p.split_size : p.N), pseq = p.N - M - first_key;
   const int m0 = mb * C::BM, mw = m0 + wave * 64;
   const int my_m[2] = {mw + l32, mw + 32 + l32};
 
   const T* qb = (const T*)p.q.ptr + batch * p.q.sb + head * p.q.sh;
-  const T* kb = (const T*)p.k.ptr + batch * p.k.sb + hk * p.k.sh;
-  const T* vb = (const T*)p.v.ptr + batch * p.v.sb + hk * p.v.sh;
+  const T* kb = (const T*)p.k.ptr + batch * p.k.sb + hk * p.k.sh + (int64_t)first_key * p.k.st;
+  const T* vb = (const T*)p.v.ptr + batch * p.v.sb + hk * p.v.sh + (int64_t)first_key * p.v.st;
 
   // ---- Q rows of this lane (one per block) as B operands: k = 16 kk + 8 hh + 0..7 ----
   V8 qreg[2][C::KSTEPS];
@@ -485,17 +491,24 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, 1) fa_fwd_wide_kernel(FwdParams p) {
     const bool empty = !(l_tot > 0.f);
     const float inv = empty ? 0.f : 1.f / l_tot;
     if (my_m[x] < M) {
-      T* ob = (T*)p.o.ptr + batch * p.o.sb + head * p.o.sh + (int64_t)my_m[x] * p.o.st;
+      const bool whole = p.num_splits <= 0;
+      const int64_t part_row = (((int64_t)batch * p.H + head) * pieces + piece) * M + my_m[x];
+      T* ob = whole ? (T*)p.o.ptr + batch * p.o.sb + head * p.o.sh + (int64_t)my_m[x] * p.o.st
+                    : (T*)((hw::half_t*)p.part_o + part_row * C::D);   // fp16 whatever T is; same element size
       static_for<16>([&](auto j_tag) {
         constexpr int db = decltype(j_tag)::value / 4, g = decltype(j_tag)::value % 4, I = 4 * x + db;
         const int d = db * 32 + 8 * g + 4 * hh;
+        const float o0 = hw::pinned_o_read<I, 4 * g + 0>(O) * inv, o1 = hw::pinned_o_read<I, 4 * g + 1>(O) * inv;
+        const float o2 = hw::pinned_o_read<I, 4 * g + 2>(O) * inv, o3 = hw::pinned_o_read<I, 4 * g + 3>(O) * inv;
         hw::u32x2 w;
-        w[0] = hw::pack2(T{}, hw::pinned_o_read<I, 4 * g + 0>(O) * inv, hw::pinned_o_read<I, 4 * g + 1>(O) * inv);
-        w[1] = hw::pack2(T{}, hw::pinned_o_read<I, 4 * g + 2>(O) * inv, hw::pinned_o_read<I, 4 * g + 3>(O) * inv);
+        w[0] = whole ? hw::pack2(T{}, o0, o1) : hw::pack2(hw::half_t{}, o0, o1);
+        w[1] = whole ? hw::pack2(T{}, o2, o3) : hw::pack2(hw::half_t{}, o2, o3);
         *(hw::u32x2*)(ob + d) = w;
       });
-      if (hh == 0)
-        p.lse[((int64_t)batch * p.H + head) * M + my_m[x]] = empty ? neg_inf() : m_ref[x] * p.sm_scale + hw::log_nat(l_tot);
+      if (hh == 0) {
+        float* lse_out = whole ? p.lse + ((int64_t)batch * p.H + head) * M + my_m[x] : p.part_lse + part_row;
+        *lse_out = empty ? neg_inf() : m_ref[x] * p.sm_scale + hw::log_nat(l_tot);
+      }
     }
   });
 }
@@ -510,10 +523,30 @@ bool fwd_wide_supported(const FwdParams& p) {
 
 int run_fwd_wide(const FwdParams& p, hipStream_t stream) {
   if (p.B <= 0 || p.H <= 0 || p.M <= 0 || p.N < 0 || p.group <= 0 || !fwd_wide_supported(p)) return kBadArgument;
-  dim3 grid(((p.M + WideCfg::BM - 1) / WideCfg::BM) * p.H * p.B, 1, 1);
+  if (p.num_splits < 0 || (p.num_splits > 0 && (p.split_size <= 0 || !p.part_o || !p.part_lse))) return kBadArgument;
+  const int pieces = p.num_splits > 0 ? p.num_splits : 1;
+  dim3 grid(((p.M + WideCfg::BM - 1) / WideCfg::BM) * p.H * p.B * pieces, 1, 1);
   if (p.dtype == kDtypeF16) return launch(fa_fwd_wide_kernel<hw::half_t>, grid, WideCfg::LDS_BYTES, stream, p);
   if (p.dtype == kDtypeBF16) return launch(fa_fwd_wide_kernel<hw::bf16_t>, grid, WideCfg::LDS_BYTES, stream, p);
   return kUnsupported;
 }
+
+// Split-KV launches with enough query rows to fill 256-row tiles run this kernel over pieces of the key axis
+// (the decode kernel behind run_splitkv serves 16 rows per workgroup).
+static FwdParams as_forward(const SplitParams& s) {
+  FwdParams p = {};
+  p.q = s.q; p.k = s.k; p.v = s.v;
+  p.B = s.B; p.H = s.H; p.M = s.M; p.N = s.N; p.D = s.D;
+  p.group = s.group; p.causal = s.causal; p.sm_scale = s.sm_scale; p.dtype = s.dtype;
+  p.num_splits = s.num_splits; p.split_size = s.split_size;
+  p.part_o = s.part_o; p.part_lse = s.part_lse;
+  return p;
+}
+
+bool splitkv_wide_applies(const SplitParams& s) {
+  return s.M >= WideCfg::BM && s.num_splits > 0 && s.split_size % WideCfg::BN == 0 && fwd_wide_supported(as_forward(s));
+}
+
+int run_splitkv_wide(const SplitParams& s, hipStream_t stream) { return run_fwd_wide(as_forward(s), stream); }
 
 }  // namespace fa

@@ -144,6 +144,7 @@ int run_splitkv(const SplitParams& p, hipStream_t stream) {
   if (p.B <= 0 || p.H <= 0 || p.M <= 0 || p.N <= 0 || p.group <= 0 || p.num_splits <= 0 || p.split_size <= 0)
     return kBadArgument;
   if ((int64_t)p.num_splits * p.split_size < p.N) return kBadArgument;
+  if (splitkv_wide_applies(p)) return run_splitkv_wide(p, stream);   // many query rows: 256-row tiles
   if (p.dtype == kDtypeF16) return launch_split<hw::half_t>(p, stream);
   if (p.dtype == kDtypeBF16) return launch_split<hw::bf16_t>(p, stream);
   return kUnsupported;

@@ -24,6 +24,12 @@ struct FwdParams {
   float dropout_p;        // 0 = no dropout; otherwise the mask is drawn from (seed, offset)
   uint64_t seed, offset;
   int block_m;            // query rows per workgroup: 128, 256, or 0 = the library's choice
+  // 256-row kernel over pieces of the key axis (0 = the whole axis, results to o / lse): piece s covers keys
+  // s * split_size .. + split_size - 1 and leaves its normalised output as fp16 in part_o (B, H, num_splits, M, D)
+  // and its log-normalizer in part_lse (B, H, num_splits, M), the layout fa_combine_kernel merges
+  int num_splits, split_size;
+  void* part_o;
+  float* part_lse;
 };
 
 struct BwdParams {
@@ -66,6 +72,9 @@ int num_cus_of_current_device();
 int run_fwd(const FwdParams& p, bool piecewise, hipStream_t stream);
 bool fwd_wide_supported(const FwdParams& p);   // the 256-row kernel (fa_fwd_wide.hip) can serve this launch
 int run_fwd_wide(const FwdParams& p, hipStream_t stream);
+struct SplitParams;
+bool splitkv_wide_applies(const SplitParams& p);   // the split-KV launch is served by the 256-row kernel
+int run_splitkv_wide(const SplitParams& p, hipStream_t stream);
 int run_bwd_delta(const BwdParams& p, hipStream_t stream);
 int run_bwd_dkdv(const BwdParams& p, bool piecewise, hipStream_t stream);
 int run_bwd_dq(const BwdParams& p, bool piecewise, hipStream_t stream);

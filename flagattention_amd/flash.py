@@ -45,6 +45,20 @@ def get_fwd_config(B, H, M, N, D, causal):
     return (128, 64, 2, 4)
 
 
+def wide_key_splits(B, H, M, N, D, num_cus):
+    """Pieces of the key axis for a dense forward launch whose 256-row workgroups (one per compute unit at a
+    time) would leave at least half of the compute units idle: Tq = 1024 against Tk = 8192 with 32 heads has
+    128 of them on 256 units.  Each piece is a workgroup of its own and the pieces are merged like the split-KV
+    path's (``split_kv.py:162-227`` of the reference); a piece keeps at least 1024 keys.  1 = do not split."""
+    if not wide_forward_applies(D) or M < 256:
+        return 1
+    wgs = -(-M // 256) * H * B
+    pieces = min(num_cus // wgs, N // 1024)
+    if pieces < 2 or 4 * pieces * wgs < 3 * num_cus:
+        return 1
+    return pieces
+
+
 _NUM_CUS = {}
 
 
@@ -123,10 +137,13 @@ class FlashAttention(torch.autograd.Function):
                 # looked up by name at call time, so that an assignment to flash.get_fwd_config takes effect
                 hook = get_fwd_config
                 block_m, _ = _config.resolve(hook, FWD_TILES, "flash_attention forward", (B, H, M, N, D, causal))
+                pieces = 1
                 if hook is _DEFAULT_FWD_CONFIG:
                     # nobody overrode the hook: the library applies the same rule and also knows what the hook
                     # is not told (dropout, the sign of sm_scale, row strides the 256-row kernel cannot address)
                     block_m = 0
+                    if not is_dropout and sm_scale > 0 and max(k.stride(2), v.stride(2)) * k.element_size() < 1 << 24:
+                        pieces = wide_key_splits(B, H, M, N, D, num_cus)
                 elif block_m == 256 and not wide_forward_applies(D, dropout_p):
                     _config.warn_once(("fwd-wide", D, is_dropout),
                                       "flash_attention forward: the 256-row kernel is built for head size 128 "
@@ -142,11 +159,14 @@ class FlashAttention(torch.autograd.Function):
                                       "flash_attention forward: the 256-row kernel addresses key/value rows less "
                                       "than 16 MiB apart; launching the 128-row kernel")
                     block_m = 128
-                o = torch.empty_like(q)
-                if not _abi.is_kernel_ready(o):
-                    o = torch.empty(q.shape, dtype=q.dtype, device=q.device)
-                L = torch.empty((B, H, M), device=q.device, dtype=torch.float32)
-                _abi.fa_fwd(lib, q, k, v, o, L, causal, sm_scale, dropout, block_m)
+                if pieces > 1:   # too few 256-row workgroups for the device: one per piece of the key axis, then the merge
+                    o, L = split_kv_forward(lib, q, k, v, causal, sm_scale, pieces, exact=True)
+                else:
+                    o = torch.empty_like(q)
+                    if not _abi.is_kernel_ready(o):
+                        o = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+                    L = torch.empty((B, H, M), device=q.device, dtype=torch.float32)
+                    _abi.fa_fwd(lib, q, k, v, o, L, causal, sm_scale, dropout, block_m)
             tot_attn = None
             if return_total_attention:
                 tot_attn = _total_attention(lib, q, k, L, causal, sm_scale)

@@ -90,13 +90,14 @@ def choose_num_splits(B, H, Hk, M, N, num_cus, reference_splits):
     return splits
 
 
-def split_kv_forward(lib, q, k, v, causal, sm_scale, splits, single_direct=False):
+def split_kv_forward(lib, q, k, v, causal, sm_scale, splits, single_direct=False, exact=False):
     """Runs the split kernel (+ merge) and returns (o, L).  ``splits`` is the count the reference's
-    rule gave; the number of pieces launched is chosen by ``choose_num_splits``.  With
+    rule gave; the number of pieces launched is chosen by ``choose_num_splits`` unless ``exact`` asks for
+    ``splits`` itself (the dense forward's own key pieces, ``flash.wide_key_splits``).  With
     ``single_direct`` a launch that ends up with one piece returns its fp16 partial output unmerged."""
     B, H, M, D = q.shape
     N = k.shape[2]
-    if splits != 1 or M <= DECODE_MAX_ROWS:
+    if not exact and (splits != 1 or M <= DECODE_MAX_ROWS):
         splits = choose_num_splits(B, H, k.shape[1], M, N, lib.fa_num_cus(), splits)
     part_lse = torch.empty((B, H, splits, M), dtype=torch.float32, device=q.device)
     part_o = torch.empty((B, H, splits, M, D), dtype=torch.float16, device=q.device)

@@ -356,3 +356,15 @@ def test_paged_attention_accepts_any_integer_context_lens_and_keeps_the_query_la
     assert name == "paged_attn_balanced" and (args[2], args[3]) == (q.stride(0), q.stride(1))
     with pytest.raises(AssertionError, match="integers"):
         flag_attn.paged_attention(q, cache, cache, torch.tensor([3., 40., 0., 17.]), table, 0.125, 40)
+
+
+def test_key_pieces_of_a_dense_forward_that_would_leave_compute_units_idle():
+    from flagattention_amd.flash import wide_key_splits
+    # (B, H, M, N, D, compute units)
+    assert wide_key_splits(1, 32, 1024, 8192, 128, 256) == 2     # 128 workgroups of 256 rows on 256 units
+    assert wide_key_splits(1, 32, 8192, 8192, 128, 256) == 1     # 1024 workgroups: nothing to gain
+    assert wide_key_splits(1, 32, 1024, 8192, 64, 256) == 1      # the 256-row kernel is built for head size 128
+    assert wide_key_splits(1, 8, 1024, 8192, 128, 256) == 8      # 32 workgroups -> 8 pieces of 1024 keys
+    assert wide_key_splits(1, 8, 1024, 4096, 128, 256) == 1      # pieces of 1024 keys would fill half the device only
+    assert wide_key_splits(1, 48, 1024, 8192, 128, 256) == 1     # 192 workgroups: a second piece would start a second round
+    assert wide_key_splits(4, 32, 100, 8192, 128, 256) == 1      # fewer rows than one 256-row tile

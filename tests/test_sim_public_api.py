@@ -205,3 +205,51 @@ def test_paged_attention_many_empty_sequences(monkeypatch, num_wgs):
     assert not out[~live].any()          # the output buffer started out as sevens
     ref = oracle_paged(q[live].float(), kc.float(), vc.float(), table[live], ctx[live], D ** -0.5)
     assert torch.allclose(out[live].float(), ref, atol=2e-3, rtol=1e-5)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_dense_forward_in_key_pieces(monkeypatch, causal):
+    """A dense launch whose 256-row workgroups would leave half the compute units idle runs the 256-row kernel
+    over pieces of the key axis and merges them (flash.wide_key_splits): the cross-length shape of the workload
+    list in small.  The last piece ends in a partial tile."""
+    B, H, Hk, M, N, D = 1, 2, 1, 300, 2100, 128
+    monkeypatch.setattr(flash, "_num_cus", lambda: 8)
+    assert flash.wide_key_splits(B, H, M, N, D, 8) == 2
+    calls = []
+    lib = _lib.get()
+
+    class Spy:
+        def __getattr__(self, name):
+            fn = getattr(lib, name)
+            if name in ("fa_fwd", "fa_splitkv_fwd", "fa_splitkv_combine"):
+                return lambda *a: (calls.append(name), fn(*a))[1]
+            return fn
+
+    monkeypatch.setattr(_lib, "get", lambda: Spy())
+    (q, k, v, do), ref, same, g_ref, g_same = flash_case(B, H, Hk, M, N, D, causal)
+    o, L, *_ = flag_attn.flash_attention(q, k, v, causal=causal, return_log_normalizer=True)
+    assert calls == ["fa_splitkv_fwd", "fa_splitkv_combine"]
+    check("o", o, same[0], ref[0])
+    check("L", L, same[1], ref[1])
+    grads = torch.autograd.grad(o, (q, k, v), do)
+    for name, h, s, r in zip(("dq", "dk", "dv"), grads, g_same, g_ref):
+        check(name, h, s, r)
+
+
+def test_key_pieces_that_some_rows_do_not_see():
+    """The split entry point with at least 256 query rows runs the 256-row kernel per piece.  Under the causal mask
+    with M = N the first row block sees nothing of the second piece: that piece reports zeros and a log-normalizer
+    of -inf for those rows and drops out of the merge."""
+    from flagattention_amd import _abi
+    lib = _lib.get()
+    B, H, M, N, D = 1, 1, 512, 512, 128
+    (q, k, v, do), ref, same, _, _ = flash_case(B, H, H, M, N, D, True, dtype=torch.float16)
+    part_o = torch.full((B, H, 2, M, D), float("nan"), dtype=torch.float16)
+    part_lse = torch.full((B, H, 2, M), float("nan"), dtype=torch.float32)
+    _abi.fa_splitkv_fwd(lib, q, k, v, part_o, part_lse, True, D ** -0.5, 2, 256)
+    assert bool((part_lse[0, 0, 1, :256] == -math.inf).all()) and not part_o[0, 0, 1, :256].any()
+    assert bool(torch.isfinite(part_lse[0, 0, 1, 256:]).all()) and bool(torch.isfinite(part_lse[0, 0, 0]).all())
+    o, L = torch.empty_like(q), torch.empty(B, H, M)
+    _abi.fa_splitkv_combine(lib, part_o, part_lse, o, L, 2)
+    check("o", o, same[0], ref[0])
+    check("L", L, same[1], ref[1])
