@@ -21,6 +21,9 @@ The JSON line also carries
   * ``other_flash_workloads``: the remaining flash configurations of the workload list as records of
     their own (B=4 H=16 T=2048; head size 64; Tq=1024 against Tk=8192), forward + backward through
     the public API;
+  * ``matrix_pipe_ceiling``: what a loop of nothing but bf16 matrix instructions reaches on the same device with
+    random and with constant operands (the device lowers its clock under a busy matrix pipe, more so the more
+    the operand bits toggle): the ceiling that applies to a kernel working on real data;
   * ``paged_decode``: the paged-attention decode configuration (64 sequences, 32 query / 8 kv heads,
     head 128, block 16, context lengths uniform in [512, 8192]) as achieved HBM GB/s;
   * ``splitkv_decode`` (dense decode over 32768 keys, three K/V sets in rotation so that no launch is
@@ -215,6 +218,23 @@ def cpu_baseline(args, torch):
                       f"fwd+bwd, best of 2, {best:.2f} s"}
 
 
+def matrix_pipe_ceiling(torch):
+    """What a loop of nothing but 32x32x16 bf16 matrix instructions reaches on this device (fa_probe_mfma: one
+    wavefront per SIMD, operands in registers), with random and with constant operands.  The clock the device
+    grants a busy matrix pipe depends on the operand values; the published peak assumes its top clock."""
+    from flagattention_amd import _abi, _lib
+    lib = _lib.get()
+    sink = torch.empty(lib.fa_num_cus() * 256, dtype=torch.float32, device="cuda:0")
+    out = {}
+    for name, rnd in (("random_operands", True), ("constant_operands", False)):
+        iters = 20000
+        flop = _abi.fa_probe_mfma(lib, sink, iters, random_operands=rnd)
+        ms = timed_launches(lambda: _abi.fa_probe_mfma(lib, sink, iters, random_operands=rnd), 3, torch, groups=3)
+        out[name] = round(flop / (ms * 1e-3) / 1e12, 1)
+    return {"kernel": "fa_probe_mfma (matrix instructions only, 1 wavefront per SIMD, bf16)", "unit": "TFLOP/s", **out,
+            "frac_of_published_peak": round(out["random_operands"] / PEAK_BF16_TFLOPS, 4)}
+
+
 def paged_bench(torch, iters=50, groups=5):
     import flagattention_amd as flag_attn
     dev = "cuda:0"
@@ -404,6 +424,7 @@ def main():
         "roofline": roofline,
         "kernels": kernels,
     }
+    out["matrix_pipe_ceiling"] = matrix_pipe_ceiling(torch)
     if not args.no_paged:
         # The other flash configurations of the workload list, as records of their own.
         legs = {"c2": (4, 16, 2048, 2048, 128), "c3": (1, 32, 8192, 8192, 128),

@@ -257,3 +257,11 @@ def paged_reduce(lib, out, tmp_out, max_logits, exp_sums, context_lens, Hkv, par
     check(lib.paged_reduce(dtype_code(out), ptr(out), out.stride(0), out.stride(1), ptr(tmp_out),
                            ptr(max_logits), ptr(exp_sums), ptr(context_lens), num_seqs, Hq, Hkv, D,
                            int(partition_size), int(num_parts), stream_of(out)), "paged_reduce")
+
+
+def fa_probe_mfma(lib, sink, iters, random_operands=True, dtype=torch.bfloat16):
+    """Enqueues the matrix-pipe rate probe on ``sink``'s device; returns the FLOP the launch executes."""
+    code = F16 if dtype == torch.float16 else BF16
+    check(lib.fa_probe_mfma(code, int(bool(random_operands)), int(iters), ptr(sink), sink.numel(), stream_of(sink)),
+          "fa_probe_mfma")
+    return lib.fa_num_cus() * 4 * int(iters) * 16 * 32768

@@ -46,6 +46,7 @@ SIGNATURES = {
     "paged_attn_balanced_workspace": [_i, _i],
     "paged_attn_balanced": [_i, _p, _i64, _i64, _p, _i64, _i64, _p, _p, _i64, _i64, _i64, _p, _p, _i, _i64,
                             _f, _i, _i, _i, _i, _i, _p, _i64, _i, _p],
+    "fa_probe_mfma": [_i, _i, _i, _p, _i64, _p],
     "paged_attn_balanced_static_prepare": [],
     "paged_attn_balanced_static": [_i, _p, _i64, _i64, _p, _i64, _i64, _p, _p, _i64, _i64, _i64, _p, _p, _i, _i64,
                                    _f, _i, _i, _i, _i, _i, _i, _p],

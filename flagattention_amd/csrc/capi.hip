@@ -429,6 +429,15 @@ int paged_attn_balanced_static(int dtype, void* out, int64_t o_stride_s, int64_t
                              num_kv_heads, head_size, block_size, ws, need, num_workgroups, stream);
 }
 
+int fa_probe_mfma(int dtype, int random_operands, int iters, float* sink, int64_t sink_floats, void* stream) {
+  const int cus = fa::num_cus_of_current_device();
+  if (cus <= 0) return FA_ERR_UNSUPPORTED;
+  if (iters <= 0 || !sink || sink_floats < (int64_t)cus * 256) return FA_ERR_BAD_ARGUMENT;
+  fa::ProbeParams p = {};
+  p.sink = sink; p.workgroups = cus; p.iters = iters; p.random_operands = random_operands; p.dtype = dtype;
+  return fa::run_probe_mfma(p, (hipStream_t)stream);
+}
+
 int paged_reduce(int dtype, void* out, int64_t o_stride_s, int64_t o_stride_h, const void* tmp_out,
                  const float* max_logits, const float* exp_sums, const int32_t* context_lens,
                  int num_seqs, int num_q_heads, int num_kv_heads, int head_size, int partition_size,

@@ -269,17 +269,54 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
     // commits its successor to LDS and then requests the tile after that
     if (t_begin + 1 < t_end) fetch((t_begin + 1) * C::BM);
 
-    // Does no mask touch the tile, so that it can run the slot-structured body?  (The same answer in
-    // every lane of a wavefront: read through a scalar register so that the loops below branch on it.)
-    auto is_plain = [&](int it) {
-      if constexpr (!FOLDED) return false;
-      const int m0 = it * C::BM;
-      // a block with keys past N goes through the masked path: its P and dS must be exact zeroes
-      // there (K and V rows are zero, so the score is just -L and exp2 of it can be huge)
-      bool plain = (nw + 31 < N) && (!p.causal || (m0 + pseq >= nw + 31));
-      // piecewise: every entry of the 64 x 32 tile belongs to this pass's regime
-      if (PW) plain = plain && (far_phase ? (m0 + pseq - (nw + 31) >= p.w) : (m0 + 63 + pseq - nw < p.w));
-      return hw::uniform((int)plain) != 0;
+    // Tiles [plain_lo, plain_hi) are touched by no mask for this wavefront's 32 keys and can run the
+    // slot-structured body (the same answer in every lane: kept in scalar registers, so that the loops below
+    // are scalar loops).  A block with keys past N goes through the masked path: its P and dS must be exact
+    // zeroes there (K and V rows are zero, so the score is just -L and exp2 of it can be huge).
+    int plain_lo = t_end, plain_hi = t_end;
+    if (FOLDED && nw + 31 < N) {
+      auto ceil64 = [](int a) { return (a + 63) >> 6; };   // also for negative a
+      plain_lo = t_begin;
+      // under the causal mask every row of the tile sees every key of the block: 64 it + pseq >= nw + 31
+      if (p.causal) plain_lo = imax(plain_lo, ceil64(nw + 31 - pseq));
+      // piecewise: every entry of the 64 x 32 tile belongs to this pass's regime --
+      // far: 64 it + pseq - (nw + 31) >= w;  near: 64 it + 63 + pseq - nw < w
+      if (PW && far_phase) plain_lo = imax(plain_lo, ceil64(p.w + nw + 31 - pseq));
+      if (PW && !far_phase) plain_hi = imin(plain_hi, ceil64(p.w + nw - 63 - pseq));
+      plain_lo = imin(plain_lo, t_end);
+      plain_hi = imax(plain_hi, plain_lo);
+    }
+    plain_lo = hw::uniform(plain_lo);
+    plain_hi = hw::uniform(plain_hi);
+    // Registers of the slot-structured body that live from one tile into the next: the score and dP accumulators
+    // of the two 32-query blocks and the ring of matrix operands read from LDS.  A tile's last slots already read
+    // the next tile's first operands and the values its first accumulator starts from, so that the first matrix
+    // instruction of a tile follows the last one of the tile before it without a trip to LDS in between.
+    f32x16 sx[2], dpx[2];
+    constexpr int kDepth = 4;
+    V8 ring[kDepth];
+    // operand of A-phase instruction j of block sb (rows of Q for j < KSTEPS, of dO behind) in the stage at `base`
+    auto a_operand_in = [&](const unsigned char* base, int sb, int j) {
+      const T* tq = (const T*)base;
+      return operand_rowmajor<T, C::LD>(j < C::KSTEPS ? tq : tq + C::TILE, sb * 32, 16 * (j % C::KSTEPS), lane);
+    };
+    auto start_scores_in = [&](const unsigned char* base, int sb) {
+      const float* tl = (const float*)(base + 2 * C::TILE * sizeof(T));
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const hw::f32x4 l4 = *(const hw::f32x4*)(tl + sb * 32 + 8 * g + 4 * hh);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sx[sb][4 * g + e] = l4[e];
+      }
+    };
+    // what a slot-structured tile expects to find when it starts: block 0's score accumulator at its rows'
+    // values and the first kDepth operands on their way (the first tile of a run; later ones get them from
+    // their predecessor's last slots)
+    auto preload = [&](int st) {
+      const unsigned char* base = smem + st * C::STAGE_BYTES;
+      start_scores_in(base, 0);
+#pragma unroll
+      for (int k = 0; k < kDepth; ++k) ring[k] = a_operand_in(base, 0, k);
     };
     // One query tile.  The two bodies are separate instantiations, run from loops of their own (below): with
     // both inside one loop the compiler carries the flags that tell them apart through every iteration and
@@ -308,7 +345,6 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
         constexpr int NA = 2 * C::KSTEPS;       // matrix instructions of an A phase (16)
         constexpr int NC = 4 * (C::DV / 32);    // of a C phase (16)
         static_assert(NA == 16 && NC == 16, "one element of a block per matrix instruction");
-        f32x16 sx[2], dpx[2];
         // operand of A-phase instruction j of block sb, and of C-phase instruction j
         auto a_operand = [&](int sb, int j) {
           return operand_rowmajor<T, C::LD>(j < C::KSTEPS ? sQ : sG, sb * 32, 16 * (j % C::KSTEPS), lane);
@@ -348,16 +384,25 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
         // element r of a block in two steps, each as early as its inputs exist, so that the element-wise
         // work spreads over as many slots as the data dependencies allow: p = exp2(c s) of block 0 from
         // the slot after its S chain ended (kP0), dS = p dP eight slots behind it, block 1 likewise a
-        // phase later; a finished pair is packed at once
+        // phase later.  The multiplications and exponentials are assembly statements that stay in their
+        // slot (left to the compiler they drift towards the matrix instruction that produced their input,
+        // closer than the hardware allows); step t multiplies element t, exponentiates element t - 1 and
+        // packs the pair that was complete a step ago, so that nothing reads an exponential in the slot
+        // that issued it.
         V8 pa[2][2], da[2][2];
         float pr[2][16];
-        float ds_prev = 0.f;
-        auto elem_p = [&](int sb, int r) {
-          pr[sb][r] = hw::exp2_fast(sx[sb][r] * c2);
-          if (r & 1) { pa[sb][r >> 3][(r & 7) - 1] = (T)pr[sb][r - 1]; pa[sb][r >> 3][r & 7] = (T)pr[sb][r]; }
+        float p_arg[2] = {0.f, 0.f}, ds_prev = 0.f;
+        auto elem_p = [&](int sb, int t) {   // t = 0 .. 17
+          if (t >= 3 && (t & 1)) {
+            const int r = t - 2;             // pair (r - 1, r), r odd
+            pa[sb][r >> 3][(r & 7) - 1] = (T)pr[sb][r - 1];
+            pa[sb][r >> 3][r & 7] = (T)pr[sb][r];
+          }
+          if (t >= 1 && t <= 16) pr[sb][t - 1] = hw::slot_exp2(p_arg[sb]);
+          if (t <= 15) p_arg[sb] = hw::slot_mul(sx[sb][t], c2);
         };
         auto elem_ds = [&](int sb, int r) {
-          const float dsv = pr[sb][r] * dpx[sb][r];
+          const float dsv = hw::slot_mul(pr[sb][r], dpx[sb][r]);
           if (r & 1) { da[sb][r >> 3][(r & 7) - 1] = (T)ds_prev; da[sb][r >> 3][r & 7] = (T)dsv; }
           ds_prev = dsv;
         };
@@ -376,12 +421,12 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
         static_assert(kD0 >= kLastDp0 + kHazardSlots, "dS of block 0 reads dP before its last product has written back");
         static_assert(kP1 >= kLastS1 + kHazardSlots, "exp2 of block 1 reads S before its last product has written back");
         static_assert(kD1 >= kLastDp1 + kHazardSlots, "dS of block 1 reads dP before its last product has written back");
-        static_assert(kD0 >= kP0 && kD1 >= kP1, "dS = p * dP needs p of the same element");
+        static_assert(kD0 > kP0 + 1 && kD1 > kP1 + 1, "dS = p * dP reads p of the same element a slot after its exponential at the earliest");
         // operands are packed in pairs as soon as their second element exists; the dV / dK products that
         // consume half block c of block sb sit in C-phase slots 8c .. 8c + 3 (dV) and 8c + 4 .. 8c + 7 (dK)
-        static_assert(kP0 + 7 < 2 * NA && kP0 + 15 < 2 * NA + 8, "P of block 0 is packed before dV takes it");
+        static_assert(kP0 + 9 < 2 * NA && kP0 + 17 < 2 * NA + 8, "P of block 0 is packed before dV takes it");
         static_assert(kD0 + 7 < 2 * NA + 4 && kD0 + 15 < 2 * NA + 12, "dS of block 0 is packed before dK takes it");
-        static_assert(kP1 + 7 < 2 * NA + NC && kP1 + 15 < 2 * NA + NC + 8, "P of block 1 is packed before dV takes it");
+        static_assert(kP1 + 9 < 2 * NA + NC && kP1 + 17 < 2 * NA + NC + 8, "P of block 1 is packed before dV takes it");
         static_assert(kD1 + 7 < 2 * NA + NC + 4 && kD1 + 15 < 2 * NA + NC + 12, "dS of block 1 is packed before dK takes it");
         // the accumulators of block 1 are re-initialised (start_scores(1) in slot NA - 6, start_dp(1) in
         // slot NA + 2) while block 1's own chains have not started and block 0's element-wise work reads
@@ -408,12 +453,12 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
         T* nG = nQ + C::TILE;
         float* nf = (float*)(nG + C::TILE);
 
-        constexpr int kDepth = 4;
-        V8 ring[kDepth];
-        start_scores(0);
-#pragma unroll
-        for (int k = 0; k < kDepth; ++k) ring[k] = operand(k);
-        start_dp(0);
+        // slots in which the tile's tail reads for its successor: the successor's stage is complete behind the
+        // barrier of slot kSyncSlot; block 0's score accumulator has been free since its last element (kP0 + 15)
+        constexpr int kNextScoresSlot = kSyncSlot + 1, kNextRingSlot = kSlots - kDepth;
+        static_assert(kNextScoresSlot > kP0 + 15 && kNextScoresSlot < kSlots && kNextRingSlot > kSyncSlot,
+                      "the next tile's first reads follow the barrier and find their registers free");
+        const unsigned char* next_base = smem + next_stage * C::STAGE_BYTES;
         hw::sched_fence();
         static_for<kSlots>([&](auto slot) {
           constexpr int k = decltype(slot)::value;
@@ -429,12 +474,15 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
                                   __builtin_bit_cast(u32x4, da[sb][c]));
           }
           if constexpr (k + kDepth < kSlots) ring[k % kDepth] = operand(k + kDepth);
+          else ring[k % kDepth] = a_operand_in(next_base, 0, k + kDepth - kSlots);   // the successor's first operands
+          if constexpr (k == 1) start_dp(0);            // needed by slot KSTEPS
+          if constexpr (k == kNextScoresSlot) start_scores_in(next_base, 0);
           if constexpr (k == NA - 6) start_scores(1);
           if constexpr (k == NA + 2) start_dp(1);
           if constexpr (k >= kD0 && k < kD0 + 16) elem_ds(0, k - kD0);
           if constexpr (k >= kD1 && k < kD1 + 16) elem_ds(1, k - kD1);
-          if constexpr (k >= kP0 && k < kP0 + 16) elem_p(0, k - kP0);
-          if constexpr (k >= kP1 && k < kP1 + 16) elem_p(1, k - kP1);
+          if constexpr (k >= kP0 && k < kP0 + 18) elem_p(0, k - kP0);
+          if constexpr (k >= kP1 && k < kP1 + 18) elem_p(1, k - kP1);
           if constexpr (k >= kCommitSlot && k < kCommitSlot + kPasses)
             qr.template commit_pass<C::LD>(nQ, k - kCommitSlot);
           if constexpr (k >= kCommitSlot + kPasses && k < kCommitSlot + 2 * kPasses)
@@ -538,14 +586,15 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
     };
     {
       int it = t_begin;
-      while (it < t_end) {
-        if constexpr (FOLDED) {
 #pragma unroll 1
-          for (; it < t_end && is_plain(it); ++it) tile(std::true_type{}, it);
-        }
+      for (; it < plain_lo; ++it) tile(std::false_type{}, it);
+      if constexpr (FOLDED) {
+        if (it < plain_hi) preload(stage);
 #pragma unroll 1
-        for (; it < t_end && !is_plain(it); ++it) tile(std::false_type{}, it);
+        for (; it < plain_hi; ++it) tile(std::true_type{}, it);
       }
+#pragma unroll 1
+      for (; it < t_end; ++it) tile(std::false_type{}, it);
     }
 
     if (PW) {  // this regime's dK is complete (piecewise has no grouped heads)

@@ -128,6 +128,16 @@ struct MaskParams {
 };
 int run_dropout_mask(const MaskParams& p, hipStream_t stream);
 
+// Matrix-pipe rate probe (probe.hip): `workgroups` workgroups of four wavefronts, each wavefront issuing
+// iters * kProbeMfmaPerIteration 32x32x16 matrix instructions from registers; sink takes one float per thread.
+constexpr int kProbeMfmaPerIteration = 16;
+struct ProbeParams {
+  float* sink;
+  int workgroups, iters, random_operands;
+  int dtype;
+};
+int run_probe_mfma(const ProbeParams& p, hipStream_t stream);
+
 int64_t bwd_ds_workspace_bytes(int B, int H, int M, int N);
 int run_bwd_dkdv_ds(const BwdParams& p, bool piecewise, hipStream_t stream);
 int run_bwd_dq_from_ds(const BwdParams& p, bool piecewise, hipStream_t stream);

@@ -247,6 +247,16 @@ int paged_attn_balanced_static(int dtype, void* out, int64_t o_stride_s, int64_t
                                int num_q_heads, int num_kv_heads, int head_size, int block_size,
                                int num_workgroups, void* stream);
 
+/* fa_probe_mfma: a measurement aid, no counterpart in the reference.  Enqueues one workgroup per compute unit
+ * (fa_num_cus() of them, 256 threads each, one wavefront per SIMD) whose wavefronts issue nothing but
+ * iters * 16 32x32x16 matrix instructions of the given dtype from registers: 2 * 32 * 32 * 16 FLOP each, so the
+ * launch executes fa_num_cus() * 4 * iters * 16 * 32768 FLOP.  With random_operands != 0 the operands are uniform
+ * in [-1, 1) and differ from lane to lane, otherwise they are a few small integers.  The caller times the launch
+ * (events on `stream`); the clock that the device grants a busy matrix pipe, and with it the rate, depends on the
+ * operand values.  sink (at least fa_num_cus() * 256 floats, sink_floats = its size) receives one float per
+ * thread and only keeps the arithmetic alive. */
+int fa_probe_mfma(int dtype, int random_operands, int iters, float* sink, int64_t sink_floats, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -372,3 +372,18 @@ def test_hand_placed_vector_instructions_of_the_256_row_forward_keep_their_dista
             assert sum(l.startswith("v_permlane32_swap") for l in lines) >= 8
             assert sum(l.startswith("v_accvgpr_write_b32") for l in lines) >= 256
     assert audited == 2
+
+
+def test_no_instruction_of_the_slotted_backward_reads_an_exponential_right_behind_it(tmp_path):
+    """The slot-structured dK/dV body issues its exponentials as assembly statements, so the compiler adds no wait
+    state between one and a reader of its result; the step order keeps them a slot apart."""
+    path = os.path.join(BUILD, "fa_bwd.o")
+    if not os.path.exists(path) or not all(shutil.which(os.path.join(LLVM, t)) for t in
+                                           ("llvm-objcopy", "clang-offload-bundler", "llvm-objdump")):
+        pytest.skip("needs the objects of a library build and the LLVM binary tools")
+    audited = 0
+    for name, lines in _disassemble(path, tmp_path).items():
+        if "fa_bwd_dkdv_kernel" in name and "Li128E" in name:
+            audited += 1
+            assert [c for c in slotted_vector_hazards(lines) if c.startswith("(b)")] == [], name
+    assert audited >= 8

@@ -479,3 +479,19 @@ def test_entry_points_reject_bad_arguments(lib):
     with pytest.raises(AssertionError):  # 3 query heads over 2 kv heads
         _abi.fa_fwd(lib, rnd((1, 3, 32, 64), torch.float16), k, k, rnd((1, 3, 32, 64), torch.float16),
                     torch.empty(1, 3, 32), False, 1.0)
+
+
+def test_matrix_pipe_probe_runs_and_fills_its_sink():
+    """The rate probe of the benchmark: one float per thread comes back; constant operands give a value that can be
+    written down -- per wavefront accumulator, iters * 4 products of A (rows (lane + e) & 3) and B (+-0.5)."""
+    from flagattention_amd import _abi
+    lib = simlib.get()
+    cus = lib.fa_num_cus()
+    sink = torch.full((cus * 256,), float("nan"))
+    flop = _abi.fa_probe_mfma(lib, sink, 1, random_operands=False)
+    assert flop == cus * 4 * 16 * 32768
+    assert bool(torch.isfinite(sink).all()) and bool((sink == sink[:256].repeat(cus)).all())
+    _abi.fa_probe_mfma(lib, sink, 1, random_operands=True)
+    assert bool(torch.isfinite(sink).all()) and sink.abs().max() > 0
+    with pytest.raises(AssertionError):
+        _abi.fa_probe_mfma(lib, sink[:10], 1)
