@@ -389,22 +389,24 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
         // closer than the hardware allows); step t multiplies element t, exponentiates element t - 1 and
         // packs the pair that was complete a step ago, so that nothing reads an exponential in the slot
         // that issued it.
-        V8 pa[2][2], da[2][2];
+        u32x4 pa[2][2], da[2][2];   // [block][half of its 16 elements]: 8 values rounded to T, the A operand of a C-phase product
         float pr[2][16];
-        float p_arg[2] = {0.f, 0.f}, ds_prev = 0.f;
+        float p_arg[2] = {0.f, 0.f};
         auto elem_p = [&](int sb, int t) {   // t = 0 .. 17
           if (t >= 3 && (t & 1)) {
             const int r = t - 2;             // pair (r - 1, r), r odd
-            pa[sb][r >> 3][(r & 7) - 1] = (T)pr[sb][r - 1];
-            pa[sb][r >> 3][r & 7] = (T)pr[sb][r];
+            pa[sb][r >> 3][(r & 7) >> 1] = hw::slot_pack2(T{}, pr[sb][r - 1], pr[sb][r]);
           }
           if (t >= 1 && t <= 16) pr[sb][t - 1] = hw::slot_exp2(p_arg[sb]);
           if (t <= 15) p_arg[sb] = hw::slot_mul(sx[sb][t], c2);
         };
-        auto elem_ds = [&](int sb, int r) {
-          const float dsv = hw::slot_mul(pr[sb][r], dpx[sb][r]);
-          if (r & 1) { da[sb][r >> 3][(r & 7) - 1] = (T)ds_prev; da[sb][r >> 3][r & 7] = (T)dsv; }
-          ds_prev = dsv;
+        float dsr[2][16];
+        auto elem_ds = [&](int sb, int t) {   // t = 0 .. 16: multiplies element t, packs the pair finished a step ago
+          if (t >= 2 && !(t & 1)) {
+            const int r = t - 1;             // pair (r - 1, r), r odd
+            da[sb][r >> 3][(r & 7) >> 1] = hw::slot_pack2(T{}, dsr[sb][r - 1], dsr[sb][r]);
+          }
+          if (t <= 15) dsr[sb][t] = hw::slot_mul(pr[sb][t], dpx[sb][t]);
         };
         constexpr int kP0 = C::KSTEPS + 1, kD0 = NA + 1, kP1 = NA + C::KSTEPS + 1, kD1 = 2 * NA + 1;
         // hw::mfma32_vacc hides its result registers from the compiler's hazard handling, so the slot
@@ -425,9 +427,11 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
         // operands are packed in pairs as soon as their second element exists; the dV / dK products that
         // consume half block c of block sb sit in C-phase slots 8c .. 8c + 3 (dV) and 8c + 4 .. 8c + 7 (dK)
         static_assert(kP0 + 9 < 2 * NA && kP0 + 17 < 2 * NA + 8, "P of block 0 is packed before dV takes it");
-        static_assert(kD0 + 7 < 2 * NA + 4 && kD0 + 15 < 2 * NA + 12, "dS of block 0 is packed before dK takes it");
+        static_assert(kD0 + 8 < 2 * NA + 4 && kD0 + 16 < 2 * NA + 12, "dS of block 0 is packed before dK takes it");
         static_assert(kP1 + 9 < 2 * NA + NC && kP1 + 17 < 2 * NA + NC + 8, "P of block 1 is packed before dV takes it");
-        static_assert(kD1 + 7 < 2 * NA + NC + 4 && kD1 + 15 < 2 * NA + NC + 12, "dS of block 1 is packed before dK takes it");
+        static_assert(kD1 + 8 < 2 * NA + NC + 4 && kD1 + 16 < 2 * NA + NC + 12, "dS of block 1 is packed before dK takes it");
+        static_assert(kD0 + 8 < 2 * NA && kD0 + 16 < 2 * NA + 8 && kD1 + 8 < 2 * NA + NC && kD1 + 16 < 2 * NA + NC + 8,
+                      "a half block of dS is packed before the slot that stores it");
         // the accumulators of block 1 are re-initialised (start_scores(1) in slot NA - 6, start_dp(1) in
         // slot NA + 2) while block 1's own chains have not started and block 0's element-wise work reads
         // only sx[0] / dpx[0]
@@ -467,11 +471,11 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
             a_issue(k / NA, k % NA, op);
           } else {
             constexpr int sb = (k - 2 * NA) / NC, j = (k - 2 * NA) % NC, c = j >> 3, db = j & 3;
-            if constexpr ((j & 4) != 0) dk[db] = hw::mfma32(da[sb][c], op, dk[db]);
-            else dv[db] = hw::mfma32(pa[sb][c], op, dv[db]);
+            if constexpr ((j & 4) != 0) dk[db] = hw::mfma32(hw::as_v8<T>(da[sb][c]), op, dk[db]);
+            else dv[db] = hw::mfma32(hw::as_v8<T>(pa[sb][c]), op, dv[db]);
             if (DS && (j & 7) == 0)
               hw::store_streaming(ds_row + (int64_t)(m0 / 32 + sb) * 1024 + c * 512,
-                                  __builtin_bit_cast(u32x4, da[sb][c]));
+                                  da[sb][c]);
           }
           if constexpr (k + kDepth < kSlots) ring[k % kDepth] = operand(k + kDepth);
           else ring[k % kDepth] = a_operand_in(next_base, 0, k + kDepth - kSlots);   // the successor's first operands
@@ -479,8 +483,8 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
           if constexpr (k == kNextScoresSlot) start_scores_in(next_base, 0);
           if constexpr (k == NA - 6) start_scores(1);
           if constexpr (k == NA + 2) start_dp(1);
-          if constexpr (k >= kD0 && k < kD0 + 16) elem_ds(0, k - kD0);
-          if constexpr (k >= kD1 && k < kD1 + 16) elem_ds(1, k - kD1);
+          if constexpr (k >= kD0 && k < kD0 + 17) elem_ds(0, k - kD0);
+          if constexpr (k >= kD1 && k < kD1 + 17) elem_ds(1, k - kD1);
           if constexpr (k >= kP0 && k < kP0 + 18) elem_p(0, k - kP0);
           if constexpr (k >= kP1 && k < kP1 + 18) elem_p(1, k - kP1);
           if constexpr (k >= kCommitSlot && k < kCommitSlot + kPasses)
