@@ -46,16 +46,21 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E peak
 # HBM traffic per launch at the default workloads, from rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE,
 # KiB per dispatch), each scaled by what the same counter reads for a plain 1 GiB device copy
 # (FETCH_SIZE reads 0.5 GiB for 1 GiB fetched -> x2.0; WRITE_SIZE reads 1.0 GiB -> x1.0);
-# profiles/hbm_traffic_dkdv_and_paged_pmc.txt.  The dK/dV and paged kernels move the same bytes as when
-# these were taken (their later changes reorder instructions and the scan of the context lengths); the
-# legs without such a measurement report traffic = null.
-DKDV_TRAFFIC_BYTES = int((2.0 * 3.631e5 + 1.0 * 1.311e5) * 1024)      # recomputing path: 744 MB read + 134 MB written
-DKDV_DS_TRAFFIC_BYTES = int((2.0 * 3.604e5 + 1.0 * 2.236e6) * 1024)   # dS kept: 738 MB read + 2.29 GB written
-PAGED_TRAFFIC_BYTES = int((2.0 * 5.014e5 + 1.0 * 4010) * 1024)        # 1.027 GB read + 4 MB written
+# profiles/hbm_traffic_per_kernel_pmc.txt holds the counter values and the commands.  Bytes.
+TRAFFIC_BYTES = {
+    "fa_fwd": 563052160,              # 256-row forward: 495 MB read + 68 MB written
+    "fa_bwd_dkdv_ds": 3033838933,     # dS kept: 744 MB read + 2.29 GB written
+    "fa_bwd_dq_from_ds": 2439147360,  # 2.37 GB read + 67 MB written
+    "paged_attn": 1031171456,          # 1.027 GB read + 4 MB written
+    "splitkv": 538585039,              # split kernel + merge
+    "piecewise": 4736987572,           # forward + delta + dK/dV (dS kept) + the two dQ-from-dS launches
+    "total_attention": 170796518,
+}
 
 WORKLOADS = {
     "c3": dict(B=1, H=32, T=8192, D=128, name="flash_attention fwd+bwd causal bf16 B=1 H=32 T=8192 D=128"),
     "c2": dict(B=4, H=16, T=2048, D=128, name="flash_attention fwd+bwd causal bf16 B=4 H=16 T=2048 D=128"),
+    "c3_d64": dict(B=1, H=32, T=8192, D=64, name="flash_attention fwd+bwd causal bf16 B=1 H=32 T=8192 D=64"),
 }
 
 
@@ -179,6 +184,8 @@ def flash_step_bench(args, torch):
         ms = timed_launches(fn, 20, torch)
         kernels[name] = {"ms": round(ms, 4), "counted_gflop": round(flops / 1e9, 2),
                          "tflops": round(flops / (ms * 1e-3) / 1e12, 1) if flops else None}
+        if args.workload == "c3" and name in TRAFFIC_BYTES:
+            kernels[name]["hbm_traffic_bytes"] = TRAFFIC_BYTES[name]
     if "fa_bwd_dq_from_ds" in kernels:   # algorithmic bytes: the visible dS blocks once, k and dq once
         ds_bytes = B * H * pairs * 2 + 2 * qd.numel() * 2
         kernels["fa_bwd_dq_from_ds"]["hbm_gbs"] = round(ds_bytes / (kernels["fa_bwd_dq_from_ds"]["ms"] * 1e-3) / 1e9, 1)
@@ -187,8 +194,8 @@ def flash_step_bench(args, torch):
     roofline = {"kernel": dkdv_name + "_kernel" if dkdv_name == "fa_bwd_dkdv" else "fa_bwd_dkdv_kernel (dS kept)",
                 "bound": "mfma", "achieved": round(achieved, 1),
                 "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
-                "traffic": None if args.workload != "c3" else
-                (DKDV_DS_TRAFFIC_BYTES if dkdv_name == "fa_bwd_dkdv_ds" else DKDV_TRAFFIC_BYTES)}
+                # measured for the default workload's dS-kept launch only
+                "traffic": TRAFFIC_BYTES["fa_bwd_dkdv_ds"] if args.workload == "c3" and dkdv_name == "fa_bwd_dkdv_ds" else None}
     step_frac = value / PEAK_BF16_TFLOPS
     return w, ms_per_step, value, roofline, kernels, step_frac
 
@@ -227,9 +234,9 @@ def matrix_pipe_ceiling(torch):
     sink = torch.empty(lib.fa_num_cus() * 256, dtype=torch.float32, device="cuda:0")
     out = {}
     for name, rnd in (("random_operands", True), ("constant_operands", False)):
-        iters = 20000
+        iters = 100000   # ~30 ms per launch: the clock needs tens of milliseconds of this load to settle
         flop = _abi.fa_probe_mfma(lib, sink, iters, random_operands=rnd)
-        ms = timed_launches(lambda: _abi.fa_probe_mfma(lib, sink, iters, random_operands=rnd), 3, torch, groups=3)
+        ms = timed_launches(lambda: _abi.fa_probe_mfma(lib, sink, iters, random_operands=rnd), 2, torch, groups=3)
         out[name] = round(flop / (ms * 1e-3) / 1e12, 1)
     return {"kernel": "fa_probe_mfma (matrix instructions only, 1 wavefront per SIMD, bf16)", "unit": "TFLOP/s", **out,
             "frac_of_published_peak": round(out["random_operands"] / PEAK_BF16_TFLOPS, 4)}
@@ -264,7 +271,7 @@ def paged_bench(torch, iters=50, groups=5):
     return {"workload": "paged_attention decode fp16 seqs=64 Hq=32 Hkv=8 D=128 block=16 ctx~U[512,8192]",
             "ms": round(ms, 4), "algorithmic_bytes": algo, "value": round(gbs, 1), "unit": "GB/s",
             "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                         "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": PAGED_TRAFFIC_BYTES}}
+                         "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": TRAFFIC_BYTES["paged_attn"]}}
 
 
 def splitkv_bench(torch, iters=48, groups=5, sets=3):
@@ -293,7 +300,7 @@ def splitkv_bench(torch, iters=48, groups=5, sets=3):
                         f"{len(sets)} K/V sets in rotation",
             "ms": round(ms, 4), "algorithmic_bytes": algo, "value": round(gbs, 1), "unit": "GB/s",
             "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                         "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None}}
+                         "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": TRAFFIC_BYTES["splitkv"]}}
 
 
 def piecewise_bench(torch, iters=10, groups=5):
@@ -315,7 +322,7 @@ def piecewise_bench(torch, iters=10, groups=5):
             "ms_fwd": round(ms_fwd, 4), "ms_bwd": round(ms_bwd, 4), "counted_gflop": round(fwd * 3.5 / 1e9, 2),
             "value": round(tf, 1), "unit": "TFLOP/s",
             "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                         "frac": round(tf / PEAK_BF16_TFLOPS, 4), "traffic": None}}
+                         "frac": round(tf / PEAK_BF16_TFLOPS, 4), "traffic": TRAFFIC_BYTES["piecewise"]}}
 
 
 def total_attention_bench(torch, iters=20, groups=5):
@@ -332,7 +339,7 @@ def total_attention_bench(torch, iters=20, groups=5):
     return {"workload": "total_attention causal bf16 B=1 H=32 T=8192 D=128", "ms": round(ms, 4),
             "counted_gflop": round(flop / 1e9, 2), "value": round(tf, 1), "unit": "TFLOP/s",
             "roofline": {"bound": "mfma", "achieved": round(tf, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                         "frac": round(tf / PEAK_BF16_TFLOPS, 4), "traffic": None}}
+                         "frac": round(tf / PEAK_BF16_TFLOPS, 4), "traffic": TRAFFIC_BYTES["total_attention"]}}
 
 
 def profile_kernel(args, torch):
@@ -348,7 +355,8 @@ def profile_kernel(args, torch):
         torch.cuda.synchronize()
         print(json.dumps({"profiled": "copy", "bytes_read": 1 << 30, "bytes_written": 1 << 30}))
         return
-    whole_legs = {"paged_attn": lambda: paged_bench(torch, iters=2, groups=1),
+    whole_legs = {"mfma_probe": lambda: matrix_pipe_ceiling(torch),
+                  "paged_attn": lambda: paged_bench(torch, iters=2, groups=1),
                   "splitkv": lambda: splitkv_bench(torch, iters=3, groups=1),
                   "piecewise": lambda: piecewise_bench(torch, iters=2, groups=1),
                   "total_attention": lambda: total_attention_bench(torch, iters=2, groups=1)}
@@ -367,7 +375,8 @@ def profile_kernel(args, torch):
     _abi.fa_fwd(lib, q, k, v, o, lse, True, sm_scale)
     _abi.fa_bwd_delta(lib, o, do, delta)
     ds = torch.empty(lib.fa_bwd_ds_workspace_mib(B, H, T, T) << 20, dtype=torch.uint8, device=dev)
-    _abi.fa_bwd_dkdv_ds(lib, q, k, v, do, lse, delta, dk, dv, ds, True, sm_scale)
+    if D == 128:   # the dS hand-over is the head-size-128 route; smaller heads recompute dS in fa_bwd_dq
+        _abi.fa_bwd_dkdv_ds(lib, q, k, v, do, lse, delta, dk, dv, ds, True, sm_scale)
     fn = {"fa_fwd": lambda: _abi.fa_fwd(lib, q, k, v, o, lse, True, sm_scale),
           "fa_bwd_dkdv": lambda: _abi.fa_bwd_dkdv(lib, q, k, v, do, lse, delta, dk, dv, True, sm_scale),
           "fa_bwd_dkdv_ds": lambda: _abi.fa_bwd_dkdv_ds(lib, q, k, v, do, lse, delta, dk, dv, ds, True, sm_scale),
@@ -394,7 +403,7 @@ def main():
     ap.add_argument("--workload", choices=sorted(WORKLOADS), default="c3")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--profile-kernel", choices=["fa_fwd", "fa_bwd_dkdv", "fa_bwd_dkdv_ds", "fa_bwd_dq", "fa_bwd_dq_from_ds",
-                                                  "paged_attn", "splitkv", "piecewise", "total_attention", "copy"],
+                                                  "paged_attn", "splitkv", "piecewise", "total_attention", "copy", "mfma_probe"],
                     help="run only this launch a few times (for rocprofv3 counter passes); 'copy' is a plain "
                          "1 GiB device copy used to calibrate FETCH_SIZE / WRITE_SIZE")
     ap.add_argument("--hold-seconds", type=float, default=0.0,
