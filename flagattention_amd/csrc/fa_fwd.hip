@@ -80,6 +80,8 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (FwdCfg<T, D, PW>::WAVES_PER_SIMD)) f
   }
 
   const float c2 = p.sm_scale * kLog2e;
+  constexpr float kLazyBits = 8.f;
+  const float lazy_tau = c2 > 0.f ? kLazyBits / c2 : 0.f;   // in units of raw scores; a non-positive scale keeps the exact maximum
   // dropout counter of (my_m, key 0)
   const uint64_t drop_row = DROP ? p.offset + (((uint64_t)batch * p.H + head) * M + (uint64_t)(my_m < M ? my_m : 0)) * N : 0;
   float m_i = neg_inf(), l_i = 0.f;
@@ -159,7 +161,12 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (FwdCfg<T, D, PW>::WAVES_PER_SIMD)) f
 #pragma unroll
       for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[nb][r]);
     mx = fmaxf(mx, hw::xor32(mx));
-    const float m_new = fmaxf(m_i, mx);
+    // The reference of the exponentials (m_i) is raised only when the tile's maximum exceeds it by more than
+    // 2^kLazyBits in the base-2 domain: softmax does not depend on the reference, probabilities up to 2^8 are
+    // exact in fp32 and in range for fp16 and bf16, and the accumulators are then rescaled a few times per
+    // row instead of in most tiles (the running maximum of 32 rows moves in every second tile of a long row).
+    const bool grow = mx > m_i + lazy_tau;   // always true for the first visible key (m_i = -inf)
+    const float m_new = grow ? mx : m_i;
     const float m_use = (m_new == neg_inf()) ? 0.f : m_new;  // row with no visible key so far
     const float shift = -m_use * c2;
     float psum = 0.f;
@@ -174,7 +181,7 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (FwdCfg<T, D, PW>::WAVES_PER_SIMD)) f
       }
     // The accumulators are rescaled only when some row of the wavefront raised its maximum;
     // after the first few tiles that is rare.
-    if (hw::wave_any(m_new > m_i)) {
+    if (hw::wave_any(grow)) {
       hw::keep_branch();
       const float alpha = hw::exp2_fast((m_i - m_use) * c2);
       l_i *= alpha;
