@@ -242,7 +242,7 @@ def matrix_pipe_ceiling(torch):
             "frac_of_published_peak": round(out["random_operands"] / PEAK_BF16_TFLOPS, 4)}
 
 
-def paged_bench(torch, iters=50, groups=5):
+def paged_bench(torch, iters=50, groups=5, zeros=False):
     import flagattention_amd as flag_attn
     dev = "cuda:0"
     g = torch.Generator(device=dev).manual_seed(10086)
@@ -261,6 +261,8 @@ def paged_bench(torch, iters=50, groups=5):
     q = torch.randn(seqs, Hq, D, device=dev, dtype=torch.float16, generator=g)
     kc = torch.randn(num_blocks, Hkv, bs, D, device=dev, dtype=torch.float16, generator=g)
     vc = torch.randn(num_blocks, Hkv, bs, D, device=dev, dtype=torch.float16, generator=g)
+    if zeros:   # same launch and traffic, operand values that toggle nothing (profile mode only)
+        q.zero_(), kc.zero_(), vc.zero_()
     scale = D ** -0.5
     fn = lambda: flag_attn.paged_attention(q, kc, vc, ctx, bt, scale, max_ctx)
     ms = timed_launches(fn, iters, torch, groups)
@@ -356,7 +358,8 @@ def profile_kernel(args, torch):
         print(json.dumps({"profiled": "copy", "bytes_read": 1 << 30, "bytes_written": 1 << 30}))
         return
     whole_legs = {"mfma_probe": lambda: matrix_pipe_ceiling(torch),
-                  "paged_attn": lambda: paged_bench(torch, iters=2, groups=1),
+                  "paged_attn": lambda: paged_bench(torch, iters=50 if args.timed else 2, groups=5 if args.timed else 1,
+                                                    zeros=args.operands == "zeros"),
                   "splitkv": lambda: splitkv_bench(torch, iters=3, groups=1),
                   "piecewise": lambda: piecewise_bench(torch, iters=2, groups=1),
                   "total_attention": lambda: total_attention_bench(torch, iters=2, groups=1)}
@@ -366,7 +369,10 @@ def profile_kernel(args, torch):
     w = WORKLOADS[args.workload]
     B, H, T, D = w["B"], w["H"], w["T"], w["D"]
     g = torch.Generator(device=dev).manual_seed(10086)
-    mk = lambda: torch.randn(B, H, T, D, device=dev, dtype=torch.bfloat16, generator=g)
+    if args.operands == "zeros":   # the same instruction stream and memory traffic on operands that toggle nothing
+        mk = lambda: torch.zeros(B, H, T, D, device=dev, dtype=torch.bfloat16)
+    else:
+        mk = lambda: torch.randn(B, H, T, D, device=dev, dtype=torch.bfloat16, generator=g)
     q, k, v, do = mk(), mk(), mk(), mk()
     sm_scale = 1.0 / math.sqrt(D)
     o, lse = torch.empty_like(q), torch.empty(B, H, T, device=dev, dtype=torch.float32)
@@ -392,7 +398,10 @@ def profile_kernel(args, torch):
             for _ in range(50):
                 fn()
             torch.cuda.synchronize()
-    print(json.dumps({"profiled": args.profile_kernel, "workload": w["name"]}))
+    out = {"profiled": args.profile_kernel, "workload": w["name"], "operands": args.operands}
+    if args.timed:
+        out["ms"] = round(timed_launches(fn, 20, torch, 5), 4)
+    print(json.dumps(out))
 
 
 def main():
@@ -408,6 +417,10 @@ def main():
                          "1 GiB device copy used to calibrate FETCH_SIZE / WRITE_SIZE")
     ap.add_argument("--hold-seconds", type=float, default=0.0,
                     help="with --profile-kernel: afterwards repeat the launch for this long")
+    ap.add_argument("--operands", choices=["random", "zeros"], default="random",
+                    help="with --profile-kernel on a flash kernel: standard-normal operands (the benchmark's) or zeros; "
+                         "the difference in time is what the device's power management takes")
+    ap.add_argument("--timed", action="store_true", help="with --profile-kernel on a flash kernel: also time the launch")
     ap.add_argument("--no-paged", action="store_true")
     ap.add_argument("--prewarm-seconds", type=float, default=0.5,
                     help="untimed steps run for this long before the counted --warmup steps (0 = none)")

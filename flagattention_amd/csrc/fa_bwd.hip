@@ -318,11 +318,22 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
 #pragma unroll
       for (int k = 0; k < kDepth; ++k) ring[k] = a_operand_in(base, 0, k);
     };
-    // One query tile.  The two bodies are separate instantiations, run from loops of their own (below): with
-    // both inside one loop the compiler carries the flags that tell them apart through every iteration and
+    // One query tile.  The bodies are separate instantiations, run from loops of their own (below): with
+    // two inside one loop the compiler carries the flags that tell them apart through every iteration and
     // allocates registers for the union of the two.
-    auto tile = [&](auto plain_tag, int it) {
-      constexpr bool plain_tile = decltype(plain_tag)::value;
+    //   kPhases       S and dP, then the element-wise work, then dV and dK, one 32 x 32 block after the other; masks
+    //                 by select, blocks that are masked as a whole skipped.  Every instantiation can run it.
+    //   kSlotsPlain   the slot-structured body for tiles that no mask touches
+    //   kSlotsMasked  the same slots with one select per element of P behind its exponential (causal mask, keys
+    //                 past N); blocks masked as a whole are computed and come out as zeroes.  Not for piecewise.
+    constexpr int kPhases = 0, kSlotsPlain = 1, kSlotsMasked = 2;
+    // first row of the tile, counted from m0, that sees key my_n (minus the 4 rows by which the upper half of the
+    // lanes is ahead in every register): element (block sb, register r) is row 32 sb + 8 (r / 4) + r % 4 + 4 hh
+    const int first_seen_row = (my_n < N ? (p.causal ? my_n - pseq : -(1 << 29)) : (1 << 29)) - 4 * hh;
+    auto tile = [&](auto kind_tag, int it) {
+      constexpr int kind = decltype(kind_tag)::value;
+      constexpr bool plain_tile = kind != kPhases;          // the slot-structured body
+      constexpr bool select_in_slots = kind == kSlotsMasked;
       const int m0 = it * C::BM;
       const bool more = it + 1 < t_end;
 
@@ -392,7 +403,13 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
         u32x4 pa[2][2], da[2][2];   // [block][half of its 16 elements]: 8 values rounded to T, the A operand of a C-phase product
         float pr[2][16];
         float p_arg[2] = {0.f, 0.f};
-        auto elem_p = [&](int sb, int t) {   // t = 0 .. 17
+        const int seen_from = first_seen_row - m0;   // rows of this tile below it are masked for this lane's key
+        auto elem_p = [&](auto sb_tag, auto t_tag) {   // t = 0 .. 17
+          constexpr int sb = decltype(sb_tag)::value, t = decltype(t_tag)::value;
+          if constexpr (select_in_slots && t >= 2) {   // element t - 2, exponentiated a step ago, before its pair is packed
+            constexpr int r = t - 2;
+            pr[sb][r] = hw::slot_keep_if_at_least<32 * sb + 8 * (r / 4) + r % 4>(pr[sb][r], seen_from);
+          }
           if (t >= 3 && (t & 1)) {
             const int r = t - 2;             // pair (r - 1, r), r odd
             pa[sb][r >> 3][(r & 7) >> 1] = hw::slot_pack2(T{}, pr[sb][r - 1], pr[sb][r]);
@@ -463,9 +480,26 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
         static_assert(kNextScoresSlot > kP0 + 15 && kNextScoresSlot < kSlots && kNextRingSlot > kSyncSlot,
                       "the next tile's first reads follow the barrier and find their registers free");
         const unsigned char* next_base = smem + next_stage * C::STAGE_BYTES;
+        // LDS accesses a slot issues: the reads of the operand kDepth slots ahead (one 16-byte read for an A-phase
+        // operand, also the successor's; two transposing reads for a C-phase operand) and whatever else is
+        // placed in it (sl < 0: a slot of the tile before)
+        auto lds_accesses_of = [](int sl) constexpr {
+          if (sl < 0) sl += kSlots;
+          const int ahead = sl + kDepth;
+          int n = (ahead >= 2 * NA && ahead < kSlots) ? 2 : 1;
+          if (sl == 1 || sl == NA - 6 || sl == NA + 2 || sl == kNextScoresSlot) n += 4;   // per-row starting values
+          if (sl >= kCommitSlot && sl <= kCommitSlot + 2 * kPasses) n += 1;              // the successor's rows
+          return n;
+        };
         hw::sched_fence();
         static_for<kSlots>([&](auto slot) {
           constexpr int k = decltype(slot)::value;
+          // one wait per pair of slots: an even slot waits for its own operand and for the next slot's, i.e. until
+          // only the accesses of the last two slots are outstanding, and the odd slot finds its operand complete
+          if constexpr ((k & 1) == 0) {
+            hw::wait_lds_pending<lds_accesses_of(k - 2) + lds_accesses_of(k - 1)>();
+            hw::sched_fence();   // or the scheduler lifts the matrix instruction over the wait and the compiler adds one of its own
+          }
           const V8 op = ring[k % kDepth];
           if constexpr (k < 2 * NA) {
             a_issue(k / NA, k % NA, op);
@@ -485,8 +519,8 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
           if constexpr (k == NA + 2) start_dp(1);
           if constexpr (k >= kD0 && k < kD0 + 17) elem_ds(0, k - kD0);
           if constexpr (k >= kD1 && k < kD1 + 17) elem_ds(1, k - kD1);
-          if constexpr (k >= kP0 && k < kP0 + 18) elem_p(0, k - kP0);
-          if constexpr (k >= kP1 && k < kP1 + 18) elem_p(1, k - kP1);
+          if constexpr (k >= kP0 && k < kP0 + 18) elem_p(std::integral_constant<int, 0>{}, std::integral_constant<int, k - kP0>{});
+          if constexpr (k >= kP1 && k < kP1 + 18) elem_p(std::integral_constant<int, 1>{}, std::integral_constant<int, k - kP1>{});
           if constexpr (k >= kCommitSlot && k < kCommitSlot + kPasses)
             qr.template commit_pass<C::LD>(nQ, k - kCommitSlot);
           if constexpr (k >= kCommitSlot + kPasses && k < kCommitSlot + 2 * kPasses)
@@ -588,17 +622,27 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
       if constexpr (!fetched_in_slots) { if (it + 2 < t_end) fetch(m0 + 2 * C::BM); }
       stage = next_stage;
     };
-    {
+    using Phases = std::integral_constant<int, kPhases>;
+    using SlotsPlain = std::integral_constant<int, kSlotsPlain>;
+    using SlotsMasked = std::integral_constant<int, kSlotsMasked>;
+    if constexpr (FOLDED && !PW) {   // every tile in slots: the masked ones (the first of the range, under the causal mask) with selects
+      int it = t_begin;
+      if (it < t_end) preload(stage);
+#pragma unroll 1
+      for (; it < plain_lo; ++it) tile(SlotsMasked{}, it);
+#pragma unroll 1
+      for (; it < t_end; ++it) tile(SlotsPlain{}, it);
+    } else {
       int it = t_begin;
 #pragma unroll 1
-      for (; it < plain_lo; ++it) tile(std::false_type{}, it);
+      for (; it < plain_lo; ++it) tile(Phases{}, it);
       if constexpr (FOLDED) {
         if (it < plain_hi) preload(stage);
 #pragma unroll 1
-        for (; it < plain_hi; ++it) tile(std::true_type{}, it);
+        for (; it < plain_hi; ++it) tile(SlotsPlain{}, it);
       }
 #pragma unroll 1
-      for (; it < t_end; ++it) tile(std::false_type{}, it);
+      for (; it < t_end; ++it) tile(Phases{}, it);
     }
 
     if (PW) {  // this regime's dK is complete (piecewise has no grouped heads)

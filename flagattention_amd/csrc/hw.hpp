@@ -181,6 +181,14 @@ FA_DEVICE uint32_t lds_address(const void* p) {
 // loads of loop-invariant operands and a loop that also prefetches: otherwise the compiler puts the
 // wait at the operands' first use INSIDE the loop, where it also covers the prefetch just issued.
 FA_DEVICE void wait_global_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // vmcnt(0), others unconstrained
+// Waits until at most N of the LDS accesses issued so far are still outstanding (they complete in order).  The
+// compiler places such waits itself, one in front of every first use of a read's result; an explicit one that
+// covers the reads of two consumers lets it drop the second's.
+template <int N>
+FA_DEVICE void wait_lds_pending() {
+  static_assert(N >= 0 && N <= 15, "the counter has four bits");
+  __builtin_amdgcn_s_waitcnt(0xC07F | (N << 8));   // lgkmcnt(N), vmcnt and expcnt unconstrained
+}
 
 // Marks a branch body as not speculatable, so that a wavefront-uniform `if` stays a branch instead
 // of being turned into unconditional arithmetic on selected operands.
@@ -245,6 +253,14 @@ FA_DEVICE float slot_max2(float a, float b) {
   return r;
 }
 FA_DEVICE void slot_add(float& acc, float x) { asm volatile("v_add_f32 %0, %0, %1" : "+v"(acc) : "v"(x)); }
+// x where bound <= C, else 0 (a select, so that an infinite x leaves no NaN); C an inline integer constant.
+// Writes vcc.  x must not be the result of the instruction right before (the compiler adds no wait state here).
+template <int C>
+FA_DEVICE float slot_keep_if_at_least(float x, int bound) {
+  static_assert(C >= -16 && C <= 64, "inline constant");
+  asm volatile("v_cmp_ge_i32 vcc, %2, %1\n\tv_cndmask_b32 %0, 0, %0, vcc" : "+v"(x) : "v"(bound), "n"(C) : "vcc");
+  return x;
+}
 FA_DEVICE uint32_t slot_pack2(half_t, float a, float b) {
   uint32_t r;
   asm volatile("v_cvt_pk_f16_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));

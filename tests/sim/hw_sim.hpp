@@ -246,6 +246,8 @@ inline int block_z() { return hwsim::bz; }
 inline void store_streaming(void* p, u32x4 v) { *(u32x4*)p = v; }
 inline u32x4 load_streaming(const void* p) { return *(const u32x4*)p; }
 inline void wait_global_loads() {}
+template <int N>
+inline void wait_lds_pending() {}
 inline int uniform(int x) { return x; }
 inline int grid_z() { return hwsim::gz; }
 inline void block_sync() { hwsim::yield(hwsim::OP_BARRIER); }
@@ -388,6 +390,8 @@ inline float slot_exp2(float x) { return exp2f(x); }
 inline float slot_max3(float a, float b, float c) { return fmaxf(fmaxf(a, b), c); }
 inline float slot_max2(float a, float b) { return fmaxf(a, b); }
 inline void slot_add(float& acc, float x) { acc += x; }
+template <int C>
+inline float slot_keep_if_at_least(float x, int bound) { return bound <= C ? x : 0.f; }
 inline uint32_t slot_pack2(half_t t, float a, float b) { return pack2(t, a, b); }
 inline uint32_t slot_pack2(bf16_t t, float a, float b) { return pack2(t, a, b); }
 
