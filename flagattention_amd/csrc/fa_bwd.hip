@@ -76,9 +76,9 @@ struct KvCfg {
   static constexpr int LD = DV + (DV == 128 ? 24 : 40);  // 16-byte row reads and transposing reads both conflict-free
   static constexpr int TILE = BM * LD;
   // register budget: two wavefronts per SIMD (256 registers each) when the accumulators allow it
-  static constexpr int WAVES_PER_SIMD = D <= 64 ? 2 : 1;
+  static constexpr int WAVES_PER_SIMD = D < 64 ? 2 : 1;
   // one wavefront per SIMD: overlap of matrix and element-wise work has to come from the instruction order
-  static constexpr bool SLOTTED = WAVES_PER_SIMD == 1 && BM == 64 && D == 128;
+  static constexpr bool SLOTTED = WAVES_PER_SIMD == 1 && BM == 64 && (D == 128 || D == 64);
   static constexpr size_t STAGE_BYTES = 2 * TILE * sizeof(T) + 2 * BM * sizeof(float);  // Q, dO, L, delta
   // the slot-structured body writes the next tile into LDS and passes the barrier before its last
   // matrix instructions, which still read the current tile: three stages
@@ -353,21 +353,23 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
       // and a scheduling fence after every such slot keeps the compiler from regrouping them.
       if constexpr (plain_tile) {
       {
-        constexpr int NA = 2 * C::KSTEPS;       // matrix instructions of an A phase (16)
-        constexpr int NC = 4 * (C::DV / 32);    // of a C phase (16)
-        static_assert(NA == 16 && NC == 16, "one element of a block per matrix instruction");
+        constexpr int NA = 2 * C::KSTEPS;       // matrix instructions of an A phase (16 at head size 128, 8 at 64)
+        constexpr int DB = C::DV / 32;          // 32-column blocks of dV and dK
+        constexpr int NC = 4 * DB;              // matrix instructions of a C phase (16 / 8)
+        static_assert(NA == NC && (NA == 16 || NA == 8), "a block's 16 elements per lane spread evenly over the slots of a phase");
+        constexpr int kRate = 16 / NA;          // elements of a block per matrix instruction
         // operand of A-phase instruction j of block sb, and of C-phase instruction j
         auto a_operand = [&](int sb, int j) {
           return operand_rowmajor<T, C::LD>(j < C::KSTEPS ? sQ : sG, sb * 32, 16 * (j % C::KSTEPS), lane);
         };
-        auto c_operand = [&](int sb, int j) {   // j = 8 c + 4 which + db
-          return operand_transposed<T, C::LD>((j & 4) ? sQ : sG, sb * 32 + 16 * (j >> 3), (j & 3) * 32, lane);
+        auto c_operand = [&](int sb, int j) {   // j = 2 DB c + DB which + db: per 16-query half c, DB products of dV, then DB of dK
+          return operand_transposed<T, C::LD>(((j / DB) & 1) ? sQ : sG, sb * 32 + 16 * (j / (2 * DB)), (j % DB) * 32, lane);
         };
         auto a_issue = [&](int sb, int j, const V8& op) {
           if (j < C::KSTEPS) sx[sb] = hw::mfma32_vacc(op, kreg[j], sx[sb]);
           else dpx[sb] = hw::mfma32_vacc(op, vreg[j - C::KSTEPS], dpx[sb]);
         };
-        // the tile's 64 matrix instructions in issue order: A0 (0-15), A1 (16-31), C0 (32-47), C1 (48-63)
+        // the tile's matrix instructions in issue order: A0, A1, C0, C1 (16 each at head size 128: slots 0-15, 16-31, 32-47, 48-63)
         constexpr int kSlots = 2 * NA + 2 * NC;
         auto operand = [&](int k) {
           if (k < NA) return a_operand(0, k);
@@ -440,19 +442,32 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
         static_assert(kD0 >= kLastDp0 + kHazardSlots, "dS of block 0 reads dP before its last product has written back");
         static_assert(kP1 >= kLastS1 + kHazardSlots, "exp2 of block 1 reads S before its last product has written back");
         static_assert(kD1 >= kLastDp1 + kHazardSlots, "dS of block 1 reads dP before its last product has written back");
-        static_assert(kD0 > kP0 + 1 && kD1 > kP1 + 1, "dS = p * dP reads p of the same element a slot after its exponential at the earliest");
-        // operands are packed in pairs as soon as their second element exists; the dV / dK products that
-        // consume half block c of block sb sit in C-phase slots 8c .. 8c + 3 (dV) and 8c + 4 .. 8c + 7 (dK)
-        static_assert(kP0 + 9 < 2 * NA && kP0 + 17 < 2 * NA + 8, "P of block 0 is packed before dV takes it");
-        static_assert(kD0 + 8 < 2 * NA + 4 && kD0 + 16 < 2 * NA + 12, "dS of block 0 is packed before dK takes it");
-        static_assert(kP1 + 9 < 2 * NA + NC && kP1 + 17 < 2 * NA + NC + 8, "P of block 1 is packed before dV takes it");
-        static_assert(kD1 + 8 < 2 * NA + NC + 4 && kD1 + 16 < 2 * NA + NC + 12, "dS of block 1 is packed before dK takes it");
-        static_assert(kD0 + 8 < 2 * NA && kD0 + 16 < 2 * NA + 8 && kD1 + 8 < 2 * NA + NC && kD1 + 16 < 2 * NA + NC + 8,
-                      "a half block of dS is packed before the slot that stores it");
-        // the accumulators of block 1 are re-initialised (start_scores(1) in slot NA - 6, start_dp(1) in
-        // slot NA + 2) while block 1's own chains have not started and block 0's element-wise work reads
-        // only sx[0] / dpx[0]
-        static_assert(NA - 6 >= 0 && NA + 2 < NA + C::KSTEPS, "block 1 starts from its rows' values before its chains run");
+        // A slot runs kRate steps of each element stream that is active in it, the dS streams before the P streams.
+        // Element r of P is final after step r + 2 of its stream (exponential in step r + 1, select in r + 2);
+        // dS of element r is step r of the dS stream.
+        constexpr auto slot_of = [](int first_slot, int step) constexpr { return first_slot + step / kRate; };
+        static_assert(slot_of(kD0, 0) > slot_of(kP0, 2) && slot_of(kD0, 15) > slot_of(kP0, 17) &&
+                      slot_of(kD1, 0) > slot_of(kP1, 2) && slot_of(kD1, 15) > slot_of(kP1, 17),
+                      "dS = p * dP reads p of the same element in a later slot than the one that finished it");
+        // operands are packed in pairs as soon as their second element exists (half c of P complete in step 8 c + 9,
+        // of dS in step 8 c + 8); half c of block sb feeds C-phase slots 2 DB c .. (dV) and 2 DB c + DB .. (dK), and
+        // the first of them also stores the half block of dS
+        constexpr auto first_dv_slot = [](int sb, int c) constexpr { return 2 * NA + sb * NC + 2 * DB * c; };
+        static_assert(slot_of(kP0, 9) < first_dv_slot(0, 0) && slot_of(kP0, 17) < first_dv_slot(0, 1) &&
+                      slot_of(kP1, 9) < first_dv_slot(1, 0) && slot_of(kP1, 17) < first_dv_slot(1, 1),
+                      "P is packed before dV takes it");
+        static_assert(slot_of(kD0, 8) < first_dv_slot(0, 0) && slot_of(kD0, 16) < first_dv_slot(0, 1) &&
+                      slot_of(kD1, 8) < first_dv_slot(1, 0) && slot_of(kD1, 16) < first_dv_slot(1, 1),
+                      "a half block of dS is packed before the slot that stores it (dK takes it DB slots later)");
+        // the accumulators of block 1 are re-initialised while block 1's own chains have not started (S: slots NA ..,
+        // dP: NA + KSTEPS ..) and after the tile before has read them for the last time (its slots up to
+        // slot_of(kP1, 15) and slot_of(kD1, 15)); block 0's likewise (start_dp(0) in slot 1, the scores in the
+        // tile before)
+        constexpr int kStartS1 = NA - 6, kStartDp1 = NA == 16 ? NA + 2 : 4;
+        static_assert(kStartS1 >= 0 && kStartS1 < NA - 2 && kStartDp1 < NA + C::KSTEPS - 1 && 1 < C::KSTEPS - 1,
+                      "a block starts from its rows' values before its chains run");
+        static_assert(slot_of(kP1, 17) < 2 * NA + 2 * NC && slot_of(kD1, 16) < 2 * NA + 2 * NC,
+                      "every element stream ends inside the tile");
 
         // The next tile's rows (in registers since the previous tile) go to the next stage during the
         // C1 slots, the workgroup's barrier follows them there, and the loads of the tile after the
@@ -464,9 +479,11 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
         // M - 1 instead of commit()'s zeroes: their P and dS are exact zeroes (L = +inf), and row M - 1
         // itself is in the same products.
         constexpr int kPasses = TileMover<T, C::BM, D>::PASSES;
-        constexpr int kCommitSlot = 2 * NA + NC, kSyncSlot = kCommitSlot + 2 * kPasses + 1;
+        // (head size 64 has 8 slots per phase: there the hand-over starts with C0, so that the barrier is passed
+        // before the last kDepth slots, which read the next tile's first operands)
+        constexpr int kCommitSlot = NA == 16 ? 2 * NA + NC : 2 * NA, kSyncSlot = kCommitSlot + 2 * kPasses + 1;
         constexpr int kFetchSlot = kCommitSlot + kPasses;   // Q registers are free from here on
-        static_assert(TileMover<T, C::BM, D>::kExact && kFetchSlot + 2 * kPasses < kSlots, "fits the C1 slots");
+        static_assert(TileMover<T, C::BM, D>::kExact && kFetchSlot + 2 * kPasses < kSlots, "fits the tile's last slots");
         const int m_ahead = imin(it + 2, t_end - 1) * C::BM;
         const T* q_ahead = q_src + (int64_t)m_ahead * q_stride;
         const T* g_ahead = gb + (int64_t)m_ahead * p.dout.st;
@@ -477,7 +494,7 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
         // slots in which the tile's tail reads for its successor: the successor's stage is complete behind the
         // barrier of slot kSyncSlot; block 0's score accumulator has been free since its last element (kP0 + 15)
         constexpr int kNextScoresSlot = kSyncSlot + 1, kNextRingSlot = kSlots - kDepth;
-        static_assert(kNextScoresSlot > kP0 + 15 && kNextScoresSlot < kSlots && kNextRingSlot > kSyncSlot,
+        static_assert(kNextScoresSlot > slot_of(kP0, 15) && kNextScoresSlot < kSlots && kNextRingSlot > kSyncSlot,
                       "the next tile's first reads follow the barrier and find their registers free");
         const unsigned char* next_base = smem + next_stage * C::STAGE_BYTES;
         // LDS accesses a slot issues: the reads of the operand kDepth slots ahead (one 16-byte read for an A-phase
@@ -487,7 +504,7 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
           if (sl < 0) sl += kSlots;
           const int ahead = sl + kDepth;
           int n = (ahead >= 2 * NA && ahead < kSlots) ? 2 : 1;
-          if (sl == 1 || sl == NA - 6 || sl == NA + 2 || sl == kNextScoresSlot) n += 4;   // per-row starting values
+          if (sl == 1 || sl == kStartS1 || sl == kStartDp1 || sl == kNextScoresSlot) n += 4;   // per-row starting values
           if (sl >= kCommitSlot && sl <= kCommitSlot + 2 * kPasses) n += 1;              // the successor's rows
           return n;
         };
@@ -504,10 +521,10 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
           if constexpr (k < 2 * NA) {
             a_issue(k / NA, k % NA, op);
           } else {
-            constexpr int sb = (k - 2 * NA) / NC, j = (k - 2 * NA) % NC, c = j >> 3, db = j & 3;
-            if constexpr ((j & 4) != 0) dk[db] = hw::mfma32(hw::as_v8<T>(da[sb][c]), op, dk[db]);
+            constexpr int sb = (k - 2 * NA) / NC, j = (k - 2 * NA) % NC, c = j / (2 * DB), db = j % DB;
+            if constexpr (((j / DB) & 1) != 0) dk[db] = hw::mfma32(hw::as_v8<T>(da[sb][c]), op, dk[db]);
             else dv[db] = hw::mfma32(hw::as_v8<T>(pa[sb][c]), op, dv[db]);
-            if (DS && (j & 7) == 0)
+            if (DS && (j % (2 * DB)) == 0)
               hw::store_streaming(ds_row + (int64_t)(m0 / 32 + sb) * 1024 + c * 512,
                                   da[sb][c]);
           }
@@ -515,12 +532,18 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
           else ring[k % kDepth] = a_operand_in(next_base, 0, k + kDepth - kSlots);   // the successor's first operands
           if constexpr (k == 1) start_dp(0);            // needed by slot KSTEPS
           if constexpr (k == kNextScoresSlot) start_scores_in(next_base, 0);
-          if constexpr (k == NA - 6) start_scores(1);
-          if constexpr (k == NA + 2) start_dp(1);
-          if constexpr (k >= kD0 && k < kD0 + 17) elem_ds(0, k - kD0);
-          if constexpr (k >= kD1 && k < kD1 + 17) elem_ds(1, k - kD1);
-          if constexpr (k >= kP0 && k < kP0 + 18) elem_p(std::integral_constant<int, 0>{}, std::integral_constant<int, k - kP0>{});
-          if constexpr (k >= kP1 && k < kP1 + 18) elem_p(std::integral_constant<int, 1>{}, std::integral_constant<int, k - kP1>{});
+          if constexpr (k == kStartS1) start_scores(1);
+          if constexpr (k == kStartDp1) start_dp(1);
+          static_for<kRate>([&](auto sub) {
+            constexpr int t0 = (k - kD0) * kRate + decltype(sub)::value, t1 = (k - kD1) * kRate + decltype(sub)::value;
+            if constexpr (k >= kD0 && t0 < 17) elem_ds(0, t0);
+            if constexpr (k >= kD1 && t1 < 17) elem_ds(1, t1);
+          });
+          static_for<kRate>([&](auto sub) {
+            constexpr int t0 = (k - kP0) * kRate + decltype(sub)::value, t1 = (k - kP1) * kRate + decltype(sub)::value;
+            if constexpr (k >= kP0 && t0 < 18) elem_p(std::integral_constant<int, 0>{}, std::integral_constant<int, (k >= kP0 ? t0 : 0)>{});
+            if constexpr (k >= kP1 && t1 < 18) elem_p(std::integral_constant<int, 1>{}, std::integral_constant<int, (k >= kP1 ? t1 : 0)>{});
+          });
           if constexpr (k >= kCommitSlot && k < kCommitSlot + kPasses)
             qr.template commit_pass<C::LD>(nQ, k - kCommitSlot);
           if constexpr (k >= kCommitSlot + kPasses && k < kCommitSlot + 2 * kPasses)
