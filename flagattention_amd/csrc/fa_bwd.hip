@@ -324,16 +324,27 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
     //   kPhases       S and dP, then the element-wise work, then dV and dK, one 32 x 32 block after the other; masks
     //                 by select, blocks that are masked as a whole skipped.  Every instantiation can run it.
     //   kSlotsPlain   the slot-structured body for tiles that no mask touches
-    //   kSlotsMasked  the same slots with one select per element of P behind its exponential (causal mask, keys
-    //                 past N); blocks masked as a whole are computed and come out as zeroes.  Not for piecewise.
-    constexpr int kPhases = 0, kSlotsPlain = 1, kSlotsMasked = 2;
-    // first row of the tile, counted from m0, that sees key my_n (minus the 4 rows by which the upper half of the
-    // lanes is ahead in every register): element (block sb, register r) is row 32 sb + 8 (r / 4) + r % 4 + 4 hh
-    const int first_seen_row = (my_n < N ? (p.causal ? my_n - pseq : -(1 << 29)) : (1 << 29)) - 4 * hh;
+    //   kSlotsMasked  the same slots with one select per element of P behind its exponential, for a mask that begins
+    //                 inside the tile: rows from a per-lane bound on are kept (causal mask, keys past N); blocks
+    //                 masked as a whole are computed and come out as zeroes
+    //   kSlotsBand    likewise with two selects per element, for the regimes of piecewise attention: rows from one
+    //                 per-lane bound up to another are kept
+    constexpr int kPhases = 0, kSlotsPlain = 1, kSlotsMasked = 2, kSlotsBand = 3;
+    // Per-lane bounds of those masks as rows counted from row 0 (the tile subtracts its m0), minus the 4 rows by
+    // which the upper half of the lanes is ahead in every register: element (block sb, register r) is row
+    // 32 sb + 8 (r / 4) + r % 4 + 4 hh.  first_seen_row: first row that sees key my_n under the causal mask;
+    // first_far_row: first row whose distance to key my_n reaches the piecewise threshold.  A key past N is seen
+    // by no row.
+    constexpr int kNoRow = 1 << 29;
+    const int first_seen_row = (my_n < N ? (p.causal ? my_n - pseq : -kNoRow) : kNoRow) - 4 * hh;
+    const int first_far_row = PW ? my_n + imax(-kNoRow, imin(p.w, kNoRow)) - pseq - 4 * hh : 0;
+    // rows [keep_from, keep_below) of this pass's regime: far = visible and at least the threshold away
+    const int keep_from = (PW && far_phase) ? imax(first_far_row, first_seen_row) : first_seen_row;
+    const int keep_below = (PW && !far_phase) ? first_far_row : kNoRow;
     auto tile = [&](auto kind_tag, int it) {
       constexpr int kind = decltype(kind_tag)::value;
       constexpr bool plain_tile = kind != kPhases;          // the slot-structured body
-      constexpr bool select_in_slots = kind == kSlotsMasked;
+      constexpr bool select_in_slots = kind == kSlotsMasked || kind == kSlotsBand;
       const int m0 = it * C::BM;
       const bool more = it + 1 < t_end;
 
@@ -405,12 +416,14 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
         u32x4 pa[2][2], da[2][2];   // [block][half of its 16 elements]: 8 values rounded to T, the A operand of a C-phase product
         float pr[2][16];
         float p_arg[2] = {0.f, 0.f};
-        const int seen_from = first_seen_row - m0;   // rows of this tile below it are masked for this lane's key
+        // the rows of this tile at which this lane's mask begins and (kSlotsBand) ends
+        const int mask_row = keep_from - m0, mask_end = keep_below - m0;
         auto elem_p = [&](auto sb_tag, auto t_tag) {   // t = 0 .. 17
           constexpr int sb = decltype(sb_tag)::value, t = decltype(t_tag)::value;
           if constexpr (select_in_slots && t >= 2) {   // element t - 2, exponentiated a step ago, before its pair is packed
             constexpr int r = t - 2;
-            pr[sb][r] = hw::slot_keep_if_at_least<32 * sb + 8 * (r / 4) + r % 4>(pr[sb][r], seen_from);
+            pr[sb][r] = hw::slot_keep_if_at_least<32 * sb + 8 * (r / 4) + r % 4>(pr[sb][r], mask_row);
+            if constexpr (kind == kSlotsBand) pr[sb][r] = hw::slot_keep_if_below<32 * sb + 8 * (r / 4) + r % 4>(pr[sb][r], mask_end);
           }
           if (t >= 3 && (t & 1)) {
             const int r = t - 2;             // pair (r - 1, r), r odd
@@ -648,24 +661,22 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
     using Phases = std::integral_constant<int, kPhases>;
     using SlotsPlain = std::integral_constant<int, kSlotsPlain>;
     using SlotsMasked = std::integral_constant<int, kSlotsMasked>;
-    if constexpr (FOLDED && !PW) {   // every tile in slots: the masked ones (the first of the range, under the causal mask) with selects
+    using SlotsBand = std::integral_constant<int, kSlotsBand>;
+    if constexpr (FOLDED) {   // every tile in slots; the ones a mask crosses (before and behind the plain range) with selects
+      using Crossed = std::conditional_t<PW, SlotsBand, SlotsMasked>;
       int it = t_begin;
       if (it < t_end) preload(stage);
 #pragma unroll 1
-      for (; it < plain_lo; ++it) tile(SlotsMasked{}, it);
+      for (; it < plain_lo; ++it) tile(Crossed{}, it);
 #pragma unroll 1
-      for (; it < t_end; ++it) tile(SlotsPlain{}, it);
-    } else {
-      int it = t_begin;
+      for (; it < plain_hi; ++it) tile(SlotsPlain{}, it);
+      if constexpr (PW) {   // (without regimes the plain range runs to the end)
 #pragma unroll 1
-      for (; it < plain_lo; ++it) tile(Phases{}, it);
-      if constexpr (FOLDED) {
-        if (it < plain_hi) preload(stage);
-#pragma unroll 1
-        for (; it < plain_hi; ++it) tile(SlotsPlain{}, it);
+        for (; it < t_end; ++it) tile(Crossed{}, it);
       }
+    } else {
 #pragma unroll 1
-      for (; it < t_end; ++it) tile(Phases{}, it);
+      for (int it = t_begin; it < t_end; ++it) tile(Phases{}, it);
     }
 
     if (PW) {  // this regime's dK is complete (piecewise has no grouped heads)

@@ -261,6 +261,13 @@ FA_DEVICE float slot_keep_if_at_least(float x, int bound) {
   asm volatile("v_cmp_ge_i32 vcc, %2, %1\n\tv_cndmask_b32 %0, 0, %0, vcc" : "+v"(x) : "v"(bound), "n"(C) : "vcc");
   return x;
 }
+// x where C < bound, else 0: the same for a mask that ends inside the tile.
+template <int C>
+FA_DEVICE float slot_keep_if_below(float x, int bound) {
+  static_assert(C >= -16 && C <= 64, "inline constant");
+  asm volatile("v_cmp_lt_i32 vcc, %2, %1\n\tv_cndmask_b32 %0, 0, %0, vcc" : "+v"(x) : "v"(bound), "n"(C) : "vcc");
+  return x;
+}
 FA_DEVICE uint32_t slot_pack2(half_t, float a, float b) {
   uint32_t r;
   asm volatile("v_cvt_pk_f16_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));

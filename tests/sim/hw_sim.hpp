@@ -392,6 +392,8 @@ inline float slot_max2(float a, float b) { return fmaxf(a, b); }
 inline void slot_add(float& acc, float x) { acc += x; }
 template <int C>
 inline float slot_keep_if_at_least(float x, int bound) { return bound <= C ? x : 0.f; }
+template <int C>
+inline float slot_keep_if_below(float x, int bound) { return C < bound ? x : 0.f; }
 inline uint32_t slot_pack2(half_t t, float a, float b) { return pack2(t, a, b); }
 inline uint32_t slot_pack2(bf16_t t, float a, float b) { return pack2(t, a, b); }
 

@@ -388,3 +388,22 @@ def test_no_instruction_of_the_slotted_backward_reads_an_exponential_right_behin
             assert [c for c in slotted_vector_hazards(lines) if c.startswith("(b)")] == [], name
             assert sum(l.startswith("v_exp_f32") for l in lines) >= 32
     assert audited >= 16
+
+
+@pytest.mark.parametrize("obj,kernel", [("fa_fwd_wide.o", "fa_fwd_wide_kernel"), ("fa_bwd.o", "fa_bwd_dkdv_kernel")])
+def test_hand_slotted_kernels_spill_nothing(obj, kernel, tmp_path):
+    """A spill is a memory instruction of the compiler's that reads a register wherever the allocator ran out: behind
+    a matrix instruction written as assembly it would read the result without the wait states (the compiler does
+    not know what the statement wrote), and in a slot it would cost what the slot was meant to hide.  The slotted
+    kernels are built so that nothing spills; a change that makes the allocator spill must show up here."""
+    path = os.path.join(BUILD, obj)
+    if not os.path.exists(path) or not all(shutil.which(os.path.join(LLVM, t)) for t in
+                                           ("llvm-objcopy", "clang-offload-bundler", "llvm-objdump")):
+        pytest.skip("needs the objects of a library build and the LLVM binary tools")
+    audited = 0
+    for name, lines in _disassemble(path, tmp_path).items():
+        if kernel in name:
+            audited += 1
+            spills = [l for l in lines if l.startswith(("scratch_", "buffer_store", "buffer_load"))]
+            assert spills == [], f"{name}: {len(spills)} scratch accesses, e.g. {spills[0]}"
+    assert audited >= 2

@@ -291,6 +291,12 @@ PW_CASES = [
     (1, 1, 330, 70, 32, 129, False, torch.float16),     # M > N, threshold on a block edge
     (2, 2, 200, 330, 128, 64, True, torch.bfloat16),    # head size 128, threshold on a block edge, two heads
     (1, 1, 270, 300, 128, 200, False, torch.bfloat16),  # head size 128: whole tiles in the near regime, and in the far one
+    # thresholds of 95 and more with head sizes 128 and 64: every tile of the backward in slots, the ones a regime
+    # begins or ends in with one select per element
+    (1, 2, 330, 330, 128, 100, True, torch.bfloat16),
+    (1, 1, 300, 400, 64, 130, True, torch.float16),
+    (1, 1, 260, 300, 64, 95, False, torch.bfloat16),
+    (1, 1, 330, 290, 128, 95, True, torch.float16),     # M > N, key tail block beside blocks in slots
 ]
 
 
