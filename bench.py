@@ -48,13 +48,13 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E peak
 # (FETCH_SIZE reads 0.5 GiB for 1 GiB fetched -> x2.0; WRITE_SIZE reads 1.0 GiB -> x1.0);
 # profiles/hbm_traffic_per_kernel_pmc.txt holds the counter values and the commands.  Bytes.
 TRAFFIC_BYTES = {
-    "fa_fwd": 563052160,              # 256-row forward: 495 MB read + 68 MB written
-    "fa_bwd_dkdv_ds": 3033838933,     # dS kept: 744 MB read + 2.29 GB written
-    "fa_bwd_dq_from_ds": 2439147360,  # 2.37 GB read + 67 MB written
-    "paged_attn": 1031171456,          # 1.027 GB read + 4 MB written
-    "splitkv": 538585039,              # split kernel + merge
-    "piecewise": 4736987572,           # forward + delta + dK/dV (dS kept) + the two dQ-from-dS launches
-    "total_attention": 170796518,
+    "fa_fwd": 566863713,              # 256-row forward: 499 MB read + 68 MB written
+    "fa_bwd_dkdv_ds": 3058307985,     # dS kept: 743 MB read + 2.32 GB written
+    "fa_bwd_dq_from_ds": 2430783746,  # 2.36 GB read + 67 MB written
+    "paged_attn": 1031160173,          # 1.027 GB read + 4 MB written
+    "splitkv": 538571646,              # split kernel + merge
+    "piecewise": 4786597015,           # forward + delta + dK/dV (dS kept) + the two dQ-from-dS launches
+    "total_attention": 170694858,
 }
 
 WORKLOADS = {
