@@ -75,7 +75,8 @@ struct KvCfg {
   static constexpr int KSTEPS = D / 16;
   static constexpr int LD = DV + (DV == 128 ? 24 : 40);  // 16-byte row reads and transposing reads both conflict-free
   static constexpr int TILE = BM * LD;
-  // register budget: two wavefronts per SIMD (256 registers each) when the accumulators allow it
+  // register budget the compiler may use: 256 registers (two wavefronts per SIMD) at the small head sizes; at 64
+  // and 128 the slot-structured body gets all 512 (at 64 it needs 229, so two workgroups still share a CU)
   static constexpr int WAVES_PER_SIMD = D < 64 ? 2 : 1;
   // one wavefront per SIMD: overlap of matrix and element-wise work has to come from the instruction order
   static constexpr bool SLOTTED = WAVES_PER_SIMD == 1 && BM == 64 && (D == 128 || D == 64);
@@ -269,10 +270,10 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
     // commits its successor to LDS and then requests the tile after that
     if (t_begin + 1 < t_end) fetch((t_begin + 1) * C::BM);
 
-    // Tiles [plain_lo, plain_hi) are touched by no mask for this wavefront's 32 keys and can run the
-    // slot-structured body (the same answer in every lane: kept in scalar registers, so that the loops below
-    // are scalar loops).  A block with keys past N goes through the masked path: its P and dS must be exact
-    // zeroes there (K and V rows are zero, so the score is just -L and exp2 of it can be huge).
+    // Tiles [plain_lo, plain_hi) are touched by no mask for this wavefront's 32 keys and run the slot-structured
+    // body without selects (the same answer in every lane: kept in scalar registers, so that the loops below are
+    // scalar loops).  A block with keys past N has no such tile: its P and dS must be exact zeroes for those keys
+    // (K and V rows are zero, so the score is just -L and exp2 of it can be huge).
     int plain_lo = t_end, plain_hi = t_end;
     if (FOLDED && nw + 31 < N) {
       auto ceil64 = [](int a) { return (a + 63) >> 6; };   // also for negative a
@@ -356,10 +357,10 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
       const int next_stage = stage + 1 == C::STAGES ? 0 : stage + 1;
       constexpr bool committed_in_slots = plain_tile, synced_in_slots = plain_tile, fetched_in_slots = plain_tile;
 
-      // Tiles that no mask touches (all but the one or two on the diagonal), with one wavefront per
-      // SIMD: nothing else would issue under this wavefront's matrix instructions, so the
-      // element-wise work of one 32 x 32 block is written BETWEEN the matrix instructions of the
-      // other, one element per matrix instruction, in the order
+      // The slot-structured body.  Nothing else would issue under this wavefront's matrix instructions (the
+      // launch bounds leave the kernel one wavefront per SIMD), so the element-wise work of one 32 x 32 block is
+      // written BETWEEN the matrix instructions of the other, one element per matrix instruction at head size
+      // 128 and two at head size 64, in the order
       //   A0 | A1 with E0 | C0 with E1 | C1      (A: S and dP, E: P and dS, C: dV and dK)
       // and a scheduling fence after every such slot keeps the compiler from regrouping them.
       if constexpr (plain_tile) {
