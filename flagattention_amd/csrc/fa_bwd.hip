@@ -208,20 +208,29 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (DROP ? 1 : KvCfg<T, D, PW>::WAVES_PE
   const float rp = DROP ? 1.f / (1.f - p.dropout_p) : 1.f;
   uint64_t drop_col = 0;  // dropout counter of (query 0, my_n) of the current head
 
-  // result block (keys x D): D along lanes, keys along registers
+  // Result block (32 keys x D) of a wavefront: in the accumulators D runs along the lanes and the keys along the
+  // registers, so a direct store would be 2 bytes per lane, 64 instructions per block.  The tiles in LDS are dead
+  // by then: the wavefront rounds its block into a patch there and stores it from the patch as whole rows, 16
+  // bytes per lane (8 instructions at head size 128).  Same values, same rounding.
   auto store_keys = [&](const f32x16* acc, const View4& dst, float scale) {
+    constexpr int PLD = C::DV + 8;                       // elements per patch row: 16-byte multiples, rows 4 apart in distinct banks
+    static_assert(4 * 32 * PLD * sizeof(T) <= C::LDS_BYTES && (PLD * sizeof(T)) % 16 == 0, "four patches fit the tile stages");
+    T* patch = (T*)smem + wave * 32 * PLD;
+    hw::block_sync();                                    // every wavefront has read the last operands of its last tile
+#pragma unroll
+    for (int db = 0; db < C::DV / 32; ++db)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) patch[block_row(r, hh) * PLD + db * 32 + l32] = (T)(acc[db][r] * scale);
+    hw::wave_sync();
     T* base = (T*)dst.ptr + batch * dst.sb + slice * dst.sh;
+    constexpr int CPR = C::DV / 8, RPI = 64 / CPR;       // 16-byte chunks per row, rows per store instruction
 #pragma unroll
-    for (int db = 0; db < C::DV / 32; ++db) {
-      const int d = db * 32 + l32;
-      if (d < D) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int n = nw + block_row(r, hh);
-          if (n < N) base[(int64_t)n * dst.st + d] = (T)(acc[db][r] * scale);
-        }
-      }
+    for (int i = 0; i < 32 / RPI; ++i) {
+      const int row = i * RPI + lane / CPR, d0 = (lane % CPR) * 8;
+      const int n = nw + row;
+      if (n < N && d0 < D) *(u32x4*)(base + (int64_t)n * dst.st + d0) = *(const u32x4*)(patch + row * PLD + d0);
     }
+    hw::block_sync();                                    // the patches are read out before a next pass writes tiles again
   };
 
   int stage = 0;
