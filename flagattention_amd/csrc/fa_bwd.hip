@@ -838,7 +838,11 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (QCfg<T, D, PW>::WAVES_PER_SIMD)) fa_
     }
     hw::wait_global_loads();  // Q and dO rows
 
-    for (int it = t_begin; it < t_end; ++it) {
+    // One key tile.  `plain`: no mask touches the tile for any row of this wavefront (and there is no dropout or
+    // second regime), so the body has no branch and the compiler may run the element-wise work of one 32-key block
+    // under the matrix instructions of the other.  The two variants run in loops of their own.
+    auto tile = [&](auto plain_tag, int it) {
+      constexpr bool plain = decltype(plain_tag)::value;
       const int n0 = it * C::BN;
       const bool more = it + 1 < t_end;
       if (more) fetch(n0 + C::BN);
@@ -849,8 +853,10 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (QCfg<T, D, PW>::WAVES_PER_SIMD)) fa_
 #pragma unroll
       for (int nb = 0; nb < C::BN / 32; ++nb) {
         const int nlo = n0 + nb * 32;
-        if (p.causal && (mw + 31 + pseq < nlo)) continue;  // block fully masked for this wavefront
-        if (PW && (far_phase ? (mw + 31 + pseq - nlo < p.w) : (mw + pseq - (nlo + 31) >= p.w))) continue;
+        if constexpr (!plain) {
+          if (p.causal && (mw + 31 + pseq < nlo)) continue;  // block fully masked for this wavefront
+          if (PW && (far_phase ? (mw + 31 + pseq - nlo < p.w) : (mw + pseq - (nlo + 31) >= p.w))) continue;
+        }
         f32x16 s, dp;
 #pragma unroll
         for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
@@ -862,7 +868,7 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (QCfg<T, D, PW>::WAVES_PER_SIMD)) fa_
           dp = hw::mfma32(operand_rowmajor<T, C::LD>(sV, nb * 32, 16 * kk, lane), greg[kk], dp);
         hw::sched_prefetched_operands<2 * C::KSTEPS, (C::KSTEPS >= 4 ? 4 : 2)>();
 
-        bool need_mask = (nlo + 32 > N) || (p.causal && (nlo + 31 > pseq + mw));
+        bool need_mask = !plain && ((nlo + 32 > N) || (p.causal && (nlo + 31 > pseq + mw)));
         if (PW) need_mask = need_mask || (far_phase ? (mw + pseq - (nlo + 31) < p.w) : (mw + 31 + pseq - nlo >= p.w));
         f32x16 ds;
         if (need_mask) {
@@ -898,6 +904,19 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (QCfg<T, D, PW>::WAVES_PER_SIMD)) fa_
       if (more) commit(stage ^ 1);
       hw::block_sync();
       stage ^= 1;
+    };
+    {
+      int it = t_begin;
+      if constexpr (!PW && !DROP) {
+        // tiles whose 64 keys exist and are visible to the wavefront's first row
+        int plain_end = imin(t_end, N / C::BN);
+        if (p.causal) plain_end = imin(plain_end, imax(0, mw + pseq + 1) / C::BN);
+        plain_end = hw::uniform(plain_end);
+#pragma unroll 1
+        for (; it < plain_end; ++it) tile(std::true_type{}, it);
+      }
+#pragma unroll 1
+      for (; it < t_end; ++it) tile(std::false_type{}, it);
     }
 
     store_rows((PW && far_phase) ? p.dq2 : p.dq);

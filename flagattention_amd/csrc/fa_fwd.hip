@@ -114,9 +114,11 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (FwdCfg<T, D, PW>::WAVES_PER_SIMD)) f
 
   const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
-  // One key tile; the LDS stage is a compile-time constant so that every operand address is a fixed
-  // offset from one per-lane base.
-  auto step = [&](int it, int t_end, int kStage) {
+  // One key tile.  `plain`: no mask touches the tile for any row of this wavefront, so the body has none of the
+  // mask branches and the compiler sees one basic block from the first product to the second (the rare rescale
+  // branch aside).  The two variants run in loops of their own.
+  auto step = [&](auto plain_tag, int it, int t_end, int kStage) {
+    constexpr bool plain = decltype(plain_tag)::value;
     const int n0 = it * C::BN;
     const bool more = it + 1 < t_end;
     if (more) fetch(n0 + C::BN);
@@ -126,7 +128,7 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (FwdCfg<T, D, PW>::WAVES_PER_SIMD)) f
 
     // A tile that the causal mask hides from all 32 rows of this wavefront (the last tiles of a
     // workgroup, for its upper wavefronts) only takes part in the data movement.
-    if (!(p.causal && (mw + 31 + pseq < n0))) {
+    if (plain || !(p.causal && (mw + 31 + pseq < n0))) {
     // ---- S^T = K Q^T : BN/32 blocks of (32 keys x 32 queries) ----
     // the two blocks advance together: consecutive matrix instructions never wait for each other
     f32x16 s[C::BN / 32];
@@ -140,8 +142,8 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (FwdCfg<T, D, PW>::WAVES_PER_SIMD)) f
     hw::sched_prefetched_operands<(C::BN / 32) * C::KSTEPS, (C::KSTEPS >= 4 ? 4 : C::KSTEPS)>();
 
     // ---- masks (key tail, causal, the other regime's entries) only on tiles that need them ----
-    bool need_mask = (n0 + C::BN > N) || (p.causal && (n0 + C::BN - 1 > pseq + mw));
-    if (PW) need_mask = need_mask || (far_phase ? (mw + pseq - (n0 + C::BN - 1) < p.w) : (mw + 31 + pseq - n0 >= p.w));
+    bool need_mask = !plain && ((n0 + C::BN > N) || (p.causal && (n0 + C::BN - 1 > pseq + mw)));
+    if (PW && !plain) need_mask = need_mask || (far_phase ? (mw + pseq - (n0 + C::BN - 1) < p.w) : (mw + 31 + pseq - n0 >= p.w));
     if (need_mask) {
 #pragma unroll
       for (int nb = 0; nb < C::BN / 32; ++nb)
@@ -231,10 +233,23 @@ FA_KERNEL void FA_LAUNCH_BOUNDS2(kThreads, (FwdCfg<T, D, PW>::WAVES_PER_SIMD)) f
     commit(stage);
     hw::block_sync();
     hw::wait_global_loads();  // Q rows
-    for (int it = t_begin; it < t_end; ++it) {
-      step(it, t_end, stage);
-      stage ^= 1;
+    // Tiles [plain_lo, plain_hi): complete (64 keys exist), visible to the wavefront's first row under the causal
+    // mask and, for piecewise attention, wholly inside this pass's regime for all 32 rows.
+    int plain_lo = t_begin, plain_hi = imin(t_end, N / C::BN);
+    if (p.causal) plain_hi = imin(plain_hi, imax(0, mw + pseq + 1) / C::BN);
+    if (PW) {
+      if (far_phase) plain_hi = imin(plain_hi, imax(0, mw + pseq - p.w + 1) / C::BN);   // 64 it + 63 <= mw + pseq - w
+      else plain_lo = imax(plain_lo, imax(-1, (mw + 31 + pseq - p.w) >> 6) + 1);          // 64 it > mw + 31 + pseq - w
     }
+    plain_lo = hw::uniform(imin(plain_lo, t_end));
+    plain_hi = hw::uniform(imax(plain_hi, plain_lo));
+    int it = t_begin;
+#pragma unroll 1
+    for (; it < plain_lo; ++it) { step(std::false_type{}, it, t_end, stage); stage ^= 1; }
+#pragma unroll 1
+    for (; it < plain_hi; ++it) { step(std::true_type{}, it, t_end, stage); stage ^= 1; }
+#pragma unroll 1
+    for (; it < t_end; ++it) { step(std::false_type{}, it, t_end, stage); stage ^= 1; }
   }
 
   // ---- epilogue: O = acc / l, L = m * scale + ln(l); rows that saw no key give O = 0, L = -inf ----
