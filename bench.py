@@ -92,8 +92,10 @@ def timed_launches(fn, iters, torch, groups=5):
     return means[len(means) // 2]
 
 
-def flash_step_leg(torch, B, H, Tq, Tk, D, iters=5):
-    """One more flash_attention forward + backward configuration, public API, as a small record."""
+def flash_step_leg(torch, B, H, Tq, Tk, D, iters=20):
+    """One more flash_attention forward + backward configuration, public API, as a small record.  Groups of 20
+    back-to-back calls, like the per-kernel timings: a group's first launch and its two event records cost some
+    tens of microseconds once, which groups of 5 calls of 0.1-0.3 ms each showed as 5-10 % of a call."""
     import flagattention_amd as flag_attn
     dev = "cuda:0"
     g = torch.Generator(device=dev).manual_seed(10086)
